@@ -42,6 +42,10 @@ class ForwardBatch:
     mm_idx: torch.Tensor | None = None     # int64 [M]
     mm_embeds: torch.Tensor | None = None  # [M, hidden]
 
+    # runs of the packed stream with their state slots (ops.seq.SeqMeta);
+    # built only for models that carry per-sequence state
+    seq: "object | None" = None
+
     @property
     def n_tokens(self) -> int:
         return self.input_ids.shape[0]

@@ -87,10 +87,22 @@ class LLMEngine:
             quantization=cfg.quantization,
             model_path=cfg.model,
             kv_cache_dtype=cfg.kv_cache_dtype,
+            max_num_seqs=cfg.max_num_seqs,
         )
         self.block_manager = BlockManager(self.runner.num_blocks, cfg.block_size)
+        # models with recurrent state: one state slot per live sequence, and
+        # no prefix reuse (cached key/value blocks cannot stand in for the
+        # recurrent state that produced the tokens after them)
+        self.state_manager = None
+        if self.runner.has_seq_state:
+            from .statecache import StateSlotManager
+
+            self.state_manager = StateSlotManager(self.runner.num_state_slots)
+            cfg.enable_prefix_caching = False
+        self._fixed: dict[str, Request] = {}
         self.scheduler = Scheduler(
             self.block_manager,
+            state_manager=self.state_manager,
             max_num_seqs=cfg.max_num_seqs,
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             max_model_len=cfg.max_model_len,
@@ -218,6 +230,46 @@ class LLMEngine:
                 )
             )
         return results
+
+    # ------------------------------------------------------------------
+    def step_fixed(self, entries, end=()) -> list[torch.Tensor]:
+        """One engine step over a caller-dictated batch, sampling nothing.
+
+        entries: [(request_id, next_token_ids, want)] — every listed
+        sequence runs exactly these tokens this step (a sequence is admitted
+        at its first entry; all entries form ONE packed forward, single
+        tokens of running sequences beside prompt portions of others);
+        `want` lists offsets into next_token_ids whose logits are returned.
+        end: ids finished after this step; their blocks and state slot are
+        given back. Returns one fp32 [len(want), vocab] tensor per entry.
+        """
+        chunks, want = [], {}
+        for rid, toks, w in entries:
+            req = self._fixed.get(rid)
+            if req is None:
+                req = Request(list(toks), SamplingParams(ignore_eos=True),
+                              request_id=rid)
+                self._fixed[rid] = req
+            else:
+                req.tokens.extend(toks)
+                req.num_prompt_tokens = len(req.tokens)
+            chunks.append((req, len(toks)))
+            want[rid] = list(w)
+        out = self.scheduler.schedule_fixed(chunks)
+        rows: dict[str, torch.Tensor] = {}
+        if not out.is_empty:
+            logits = self.runner.forward_logits(out, want)
+            self.step_count += 1
+            ofs = 0
+            for ss in out.all_seqs:
+                n = len(want[ss.req.request_id])
+                rows[ss.req.request_id] = logits[ofs : ofs + n]
+                ofs += n
+        ended = [self._fixed.pop(rid) for rid in end if rid in self._fixed]
+        self.scheduler.finish_fixed(out, ended)
+        for req in ended:
+            self.runner.release_request(req.request_id)
+        return [rows[rid] for rid, _, _ in entries]
 
     # ------------------------------------------------------------------
     def embed(self, tok_lists: list[list[int]]) -> list[list[float]]:

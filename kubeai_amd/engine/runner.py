@@ -14,7 +14,7 @@ import torch
 
 from kubeai_amd import ops
 from kubeai_amd.models.config import ModelArchConfig
-from kubeai_amd.models.llama import LlamaForCausalLM
+from kubeai_amd.models.registry import model_class
 
 from .batch import ForwardBatch
 from .scheduler import SchedulerOutput
@@ -98,6 +98,7 @@ class ModelRunner:
         quantization: Optional[str] = None,
         model_path: Optional[str] = None,
         kv_cache_dtype: str = "auto",
+        max_num_seqs: int = 256,
     ):
         self.arch = arch
         self.device = torch.device(device)
@@ -135,9 +136,19 @@ class ModelRunner:
             )
             self.n_kv_local = self.model.n_kv_local
         else:
-            self.model = LlamaForCausalLM(arch, device=self.device, dtype=dtype)
+            self.model = model_class(arch.architecture)(
+                arch, device=self.device, dtype=dtype
+            )
             self.n_kv_local = arch.num_key_value_heads
         self.model.eval()
+        # models with per-sequence recurrent state get a slot per live
+        # sequence (engine/statecache.py) and a SeqMeta in every batch
+        self.has_seq_state = bool(getattr(self.model, "has_seq_state", False))
+        if self.has_seq_state and tp_group is not None:
+            raise NotImplementedError(
+                "tensor parallelism is not implemented for models with "
+                "per-sequence recurrent state"
+            )
         # multimodal: the vision tower is replicated on every rank (it
         # runs once per image at prefill; TP ranks compute identical
         # embeddings deterministically instead of broadcasting them)
@@ -179,34 +190,58 @@ class ModelRunner:
             self.kv_dtype = dtype
         else:
             raise ValueError(f"unknown kv_cache_dtype {kv_cache_dtype!r}")
+        # per-layer cache shapes: (kv heads, key dim, value dim), or None for
+        # a layer that keeps no paged keys/values
+        if hasattr(self.model, "kv_cache_specs"):
+            self.kv_specs = list(self.model.kv_cache_specs())
+        else:
+            self.kv_specs = [
+                (self.n_kv_local, arch.head_dim, arch.head_dim)
+            ] * arch.num_hidden_layers
         if num_gpu_blocks is None:
             num_gpu_blocks = self._profile_num_blocks(gpu_memory_utilization)
         self.num_blocks = num_gpu_blocks
-        kv_shape = (
-            num_gpu_blocks,
-            self.n_kv_local,
-            block_size,
-            arch.head_dim,
-        )
         self.kv_caches = [
-            (
-                torch.zeros(kv_shape, dtype=self.kv_dtype, device=self.device),
-                torch.zeros(kv_shape, dtype=self.kv_dtype, device=self.device),
+            None
+            if spec is None
+            else (
+                torch.zeros(
+                    (num_gpu_blocks, spec[0], block_size, spec[1]),
+                    dtype=self.kv_dtype, device=self.device,
+                ),
+                torch.zeros(
+                    (num_gpu_blocks, spec[0], block_size, spec[2]),
+                    dtype=self.kv_dtype, device=self.device,
+                ),
             )
-            for _ in range(arch.num_hidden_layers)
+            for spec in self.kv_specs
         ]
         self.model.bind_kv_caches(self.kv_caches)
+        # recurrent / convolution state: fp32 [num_state_slots, ...] per
+        # layer run, indexed by the sequence's slot
+        self.num_state_slots = 0
+        self.states = None
+        if self.has_seq_state:
+            self.num_state_slots = max(1, int(max_num_seqs))
+            self.states = [
+                {
+                    name: torch.zeros(
+                        (self.num_state_slots,) + tuple(shape),
+                        dtype=torch.float32, device=self.device,
+                    )
+                    for name, shape in spec.items()
+                }
+                for spec in self.model.state_specs()
+            ]
+            self.model.bind_states(self.states)
 
     def _profile_num_blocks(self, gpu_memory_utilization: float) -> int:
-        per_block_bytes = (
-            2  # k + v
-            * self.n_kv_local
-            * self.block_size
-            * self.arch.head_dim
-            * self.kv_dtype.itemsize
-            * self.arch.num_hidden_layers
+        per_block_bytes = sum(
+            spec[0] * self.block_size * (spec[1] + spec[2]) * self.kv_dtype.itemsize
+            for spec in self.kv_specs
+            if spec is not None
         )
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and per_block_bytes > 0:
             free, total = torch.cuda.mem_get_info(self.device)
             budget = total * gpu_memory_utilization - (total - free)
             # reserve activation headroom: 4% of total
@@ -217,7 +252,7 @@ class ModelRunner:
                     f"not enough GPU memory for KV cache: budget={budget/1e9:.1f}GB"
                 )
             return n
-        return 512  # CPU tests
+        return 512  # CPU tests / models without paged keys
 
     # ------------------------------------------------------------------
     # LoRA (full SGMV path in kubeai_amd/engine/lora.py; ids are also the
@@ -234,7 +269,10 @@ class ModelRunner:
             self.lora_manager.unload(lora_id)
 
     # ------------------------------------------------------------------
-    def build_batch(self, out: SchedulerOutput) -> ForwardBatch:
+    def build_batch(self, out: SchedulerOutput, want=None) -> ForwardBatch:
+        """want: optional {request_id: [offsets into this step's tokens]} —
+        the rows whose logits the caller asks for, instead of the rows the
+        sampler needs (replaying a fixed token stream samples nothing)."""
         bs = self.block_size
         # vision embeddings: computed once per request, at its first
         # scheduled prefill chunk
@@ -306,11 +344,24 @@ class ModelRunner:
         # samples its last chunk token if the chunk completes the prompt
         logit_idx: list[int] = []
         nd = len(out.decode)
-        for i, ss in enumerate(out.decode):
-            logit_idx.append(i)
-        for j, ss in enumerate(out.prefill):
-            if ss.samples:
-                logit_idx.append(nd + qsl[j + 1] - 1)
+        if want is not None:
+            for i, ss in enumerate(out.decode):
+                logit_idx.extend(i + o for o in want.get(ss.req.request_id, ()))
+            for j, ss in enumerate(out.prefill):
+                logit_idx.extend(
+                    nd + qsl[j] + o for o in want.get(ss.req.request_id, ())
+                )
+        else:
+            for i, ss in enumerate(out.decode):
+                logit_idx.append(i)
+            for j, ss in enumerate(out.prefill):
+                if ss.samples:
+                    logit_idx.append(nd + qsl[j + 1] - 1)
+        # runs of the stream with their state slots, in packing order;
+        # bucket padding below appends slot-less runs
+        runs: list[tuple[int, int]] = [
+            (ss.chunk_len, ss.req.state_slot) for ss in out.all_seqs
+        ]
 
         lora_ids = None
         if getattr(self, "lora_manager", None) is not None and self.lora_manager.active:
@@ -336,6 +387,7 @@ class ModelRunner:
             while left > 0:
                 c = min(left, bs)
                 positions.extend(range(c))
+                runs.append((c, -1))
                 pre_tables.append([0] * max_bt)
                 pre_lens.append(c)
                 qsl.append(qsl[-1] + c)
@@ -348,7 +400,16 @@ class ModelRunner:
         dev = self.device
         t32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
         n_prefill = len(pre_lens)
+        seq = None
+        pos_t = t32(positions)
+        if self.has_seq_state:
+            from kubeai_amd.ops.seq import SeqMeta
+
+            seq = SeqMeta.build(
+                runs, pos_t, dev, block_tables=t32(dec_tables + pre_tables)
+            )
         return ForwardBatch(
+            seq=seq,
             mm_idx=(
                 torch.tensor(mm_idx, dtype=torch.int64, device=dev)
                 if mm_idx
@@ -357,7 +418,7 @@ class ModelRunner:
             mm_embeds=torch.cat(mm_rows).to(dev) if mm_rows else None,
             lora_ids=lora_ids,
             input_ids=t32(input_ids),
-            positions=t32(positions),
+            positions=pos_t,
             slot_mapping=torch.tensor(slots, dtype=torch.int64, device=dev),
             n_decode=nd,
             decode_block_tables=t32(dec_tables) if dec_tables else None,
@@ -429,11 +490,24 @@ class ModelRunner:
         )
 
     @torch.inference_mode()
+    def forward_logits(self, out: SchedulerOutput, want) -> torch.Tensor:
+        """One forward of the scheduled step; fp32 logits [rows, vocab] for
+        the rows named by `want` ({request_id: [offsets into the tokens the
+        request contributes this step]}), decode sequences first, then
+        prompt portions, each in scheduled order. Samples nothing."""
+        fb = self.build_batch(out, want=want)
+        hidden = self.model(fb)
+        if fb.logits_indices.numel() == 0:
+            return torch.empty((0, self.arch.vocab_size), dtype=torch.float32)
+        return self.model.compute_logits(hidden[fb.logits_indices])
+
+    @torch.inference_mode()
     def execute(self, out: SchedulerOutput, step: int) -> dict[str, int]:
         """Run one forward + sampling; returns request_id -> sampled token."""
         logits = None
         if (
             self.enable_graphs
+            and not self.has_seq_state
             and not out.prefill
             and out.decode
             and not (

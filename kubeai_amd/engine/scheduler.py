@@ -99,6 +99,9 @@ class Request:
         self.num_prompt_tokens = len(prompt_token_ids)
         self.num_computed = 0  # tokens whose KV sits in the cache
         self.block_table: list[int] = []
+        # slot of the per-sequence recurrent state (models that carry one);
+        # -1 while not admitted
+        self.state_slot: int = -1
         self.block_hashes: list[int] = []  # sealed-block hash chain
         self.num_cached_prompt_tokens = 0  # prefix-cache hits at admission
 
@@ -158,8 +161,13 @@ class Scheduler:
         max_model_len: int = 8192,
         enable_prefix_caching: bool = True,
         prefill_interval: int = 1,
+        state_manager=None,
     ):
         self.bm = block_manager
+        # StateSlotManager for models with per-sequence recurrent state: a
+        # sequence holds one slot from admission until it finishes, is
+        # aborted or is preempted
+        self.sm = state_manager
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
@@ -271,6 +279,8 @@ class Scheduler:
         ):
             req = self.waiting[0]
             n_prompt = req.num_prompt_tokens
+            if self.sm is not None and self.sm.num_free == 0:
+                break
             try:
                 table, n_cached = self.bm.allocate(
                     req.tokens[:n_prompt],
@@ -282,6 +292,8 @@ class Scheduler:
             except NoFreeBlocks:
                 break
             req.block_table = table
+            if self.sm is not None:
+                req.state_slot = self.sm.allocate(req.request_id)
             req.num_computed = n_cached
             req.num_cached_prompt_tokens = n_cached
             # rebuild the sealed-hash chain for the cached prefix
@@ -337,9 +349,16 @@ class Scheduler:
                     victim = (key, req)
         return victim[1] if victim else None
 
-    def _preempt(self, req: Request, preempted: list[Request]) -> None:
+    def _release(self, req: Request) -> None:
+        """Give back what a sequence holds: its cache blocks and state slot."""
         self.bm.free(req.block_table)
         req.block_table = []
+        if self.sm is not None and req.state_slot >= 0:
+            self.sm.free(req.state_slot)
+        req.state_slot = -1
+
+    def _preempt(self, req: Request, preempted: list[Request]) -> None:
+        self._release(req)
         req.block_hashes = []
         req.num_computed = 0
         req.status = RequestStatus.WAITING
@@ -386,10 +405,48 @@ class Scheduler:
             if req.status.finished:
                 finished.append(req)
         for req in finished:
-            self.bm.free(req.block_table)
-            req.block_table = []
+            self._release(req)
             self.running.remove(req)
         return finished
+
+    # ----------------------------------------------------------------
+    # fixed schedules: the caller dictates which sequences run and how many
+    # tokens each contributes (replaying a recorded token stream). Blocks
+    # and state slots come from the same managers as in schedule(); nothing
+    # is preempted — running out of either is the caller's error.
+    def schedule_fixed(self, chunks: list[tuple[Request, int]]) -> SchedulerOutput:
+        decode: list[ScheduledSeq] = []
+        prefill: list[ScheduledSeq] = []
+        bs = self.bm.block_size
+        for req, n in chunks:
+            if n <= 0:
+                continue
+            if req.status == RequestStatus.WAITING:
+                if len(self.running) >= self.max_num_seqs:
+                    raise RuntimeError("fixed schedule exceeds max_num_seqs")
+                if self.sm is not None:
+                    req.state_slot = self.sm.allocate(req.request_id)
+                req.block_table = []
+                req.num_computed = 0
+                req.status = RequestStatus.RUNNING
+                self.running.append(req)
+            need = req.num_computed + n
+            if need > len(req.tokens):
+                raise ValueError("fixed schedule runs past the sequence's tokens")
+            while len(req.block_table) * bs < need:
+                self.bm.append_block(req.block_table)  # NoFreeBlocks propagates
+            ss = ScheduledSeq(req, req.num_computed, n)
+            (decode if n == 1 and req.num_computed > 0 else prefill).append(ss)
+        return SchedulerOutput(decode=decode, prefill=prefill, preempted=[])
+
+    def finish_fixed(self, output: SchedulerOutput, ended: list[Request]) -> None:
+        for ss in output.all_seqs:
+            ss.req.num_computed += ss.chunk_len
+        for req in ended:
+            if req.status == RequestStatus.RUNNING:
+                req.status = RequestStatus.FINISHED_STOPPED
+                self._release(req)
+                self.running.remove(req)
 
     def _maybe_finish(self, req: Request, tok: int, now: float) -> None:
         p = req.params
@@ -408,8 +465,7 @@ class Scheduler:
         for req in list(self.running):
             if req.request_id in self._aborted:
                 req.status = RequestStatus.FINISHED_ABORTED
-                self.bm.free(req.block_table)
-                req.block_table = []
+                self._release(req)
                 self.running.remove(req)
         self.waiting = deque(
             r for r in self.waiting if r.request_id not in self._aborted

@@ -64,6 +64,10 @@ class ModelArchConfig:
     # placeholder positions at admission; models/vision.py)
     vision: dict | None = None
     image_token_id: int = -1
+    # hybrid designs (per-layer mixers: recurrences, chunked attention, ...):
+    # the list of HybridLayerSpec plus the design's scalar constants.
+    # None for the homogeneous attention families above.
+    hybrid: "HybridSpec | None" = None
 
     @property
     def n_kv_heads(self) -> int:
@@ -73,6 +77,8 @@ class ModelArchConfig:
     def from_hf_config(path: str) -> "ModelArchConfig":
         with open(os.path.join(path, "config.json")) as f:
             cfg = json.load(f)
+        if cfg.get("architecture") == "Dulotar":
+            return dulotar_arch_config(cfg)
         hidden = cfg["hidden_size"]
         n_heads = cfg["num_attention_heads"]
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
@@ -168,6 +174,60 @@ class ModelArchConfig:
             vision=vision,
             image_token_id=image_token_id,
         )
+
+
+@dataclasses.dataclass
+class HybridLayerSpec:
+    """One layer of a hybrid design: which mixer, its sizes/constants as the
+    checkpoint's config gives them, its feed-forward (None = the layer has
+    only the mixer sublayer), and the layer whose tensors it uses."""
+
+    type: str
+    mixer: dict
+    mlp: dict | None
+    weights_of: int  # own index unless the layer shares another's tensors
+
+
+@dataclasses.dataclass
+class HybridSpec:
+    layers: list
+    norm_eps: float
+    embedding_scale: float
+    canon_taps: int  # taps of the per-layer input convolution (0 = none)
+
+
+def dulotar_arch_config(cfg: dict) -> ModelArchConfig:
+    """Dulotar config.json -> arch config. Every size and constant comes
+    from the file; nothing is defaulted to a particular checkpoint."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        layers.append(
+            HybridLayerSpec(
+                type=L["type"],
+                mixer=L["mixer"],
+                mlp=L.get("mlp"),
+                weights_of=int(L.get("weights_of", i)),
+            )
+        )
+    return ModelArchConfig(
+        architecture="dulotar",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]),
+        num_hidden_layers=len(layers),
+        intermediate_size=0,
+        num_attention_heads=0,
+        num_key_value_heads=0,
+        head_dim=0,
+        max_position_embeddings=1 << 30,  # no learned/cached position table
+        bos_token_id=-1,
+        eos_token_id=-1,  # the design defines no end token
+        hybrid=HybridSpec(
+            layers=layers,
+            norm_eps=float(cfg["norm"]["eps"]),
+            embedding_scale=float(cfg["embedding"]["scale"]),
+            canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+        ),
+    )
 
 
 # Presets (BASELINE.json configs + test-size models)

@@ -277,6 +277,9 @@ def load_weights(model, model_dir: str, vision=None) -> int:
     vision: optional models/vision.py VisionTower — llava checkpoints
     route their vision_tower.* / multi_modal_projector.* tensors there
     (HF llava nests the text model under language_model.*)."""
+    if hasattr(model, "load_named_tensors"):
+        # families with their own checkpoint naming map it themselves
+        return model.load_named_tensors(iter_safetensors(model_dir))
     cfg = model.cfg
     hd, nq, nkv = cfg.head_dim, cfg.num_attention_heads, cfg.num_key_value_heads
     params = dict(model.named_parameters())

@@ -1,0 +1,260 @@
+"""Token mixers beyond plain causal attention, for hybrid layer stacks.
+
+Each mixer is parameterised by its own sizes and constants (never by a
+particular checkpoint) and declares what it carries between steps:
+
+  state_spec()  -> {name: per-slot shape}  fp32 tensors [slots, *shape]
+  kv_spec()     -> None | (kv_heads, key_dim, value_dim) for a paged cache
+
+forward() gets the activations h [T, C] of the packed step, the ForwardBatch
+(whose .seq describes the runs and their state slots), this layer's state
+tensors and paged cache. Projections are library GEMMs in the serving dtype;
+everything inside a recurrence, every norm and every attention score is fp32
+in the kernels (kubeai_amd.ops.seq).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from kubeai_amd.ops import seq as sops
+
+
+def _f32(*shape):
+    return nn.Parameter(torch.zeros(*shape, dtype=torch.float32), requires_grad=False)
+
+
+class Proj(nn.Module):
+    """Bias-free linear layer [out, in] in the serving dtype."""
+
+    def __init__(self, n_in: int, n_out: int):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(n_out, n_in), requires_grad=False)
+        nn.init.normal_(self.weight, std=n_in ** -0.5)
+
+    def forward(self, x):
+        return F.linear(x, self.weight)
+
+
+class CausalConvTails(nn.Module):
+    """Depthwise causal convolution over time whose last taps-1 inputs are
+    sequence state (the layer-input convolution and the q/k/v convolutions)."""
+
+    def __init__(self, channels: int, taps: int, residual: bool):
+        super().__init__()
+        self.taps = taps
+        self.residual = residual
+        self.weight = _f32(channels, taps)
+        nn.init.normal_(self.weight, std=0.3)
+        self.channels = channels
+
+    def state_shape(self):
+        return (self.taps - 1, self.channels)
+
+    def forward(self, x, fb, tails):
+        return sops.causal_conv(x, self.weight, tails, fb.seq, self.residual)
+
+
+class MinGRUMixer(nn.Module):
+    """minGRU: elementwise recurrent state; gate and candidate depend on the input at t alone."""
+
+    def __init__(self, width: int, n: int):
+        super().__init__()
+        self.n = n
+        self.in_proj = Proj(width, 3 * n)  # z | x | g
+        self.bias_z = _f32(n)
+        self.bias_x = _f32(n)
+        self.o_proj = Proj(n, width)
+
+    def state_spec(self):
+        return {"s": (self.n,)}
+
+    def kv_spec(self):
+        return None
+
+    def forward(self, h, fb, state, kv_cache):
+        zxg = self.in_proj(h)
+        y = sops.mingru_scan(zxg, self.bias_z, self.bias_x, state["s"], fb.seq)
+        return self.o_proj(y)
+
+
+class WKVMixer(nn.Module):
+    """Matrix-state time mixing with token shift and data-dependent
+    per-channel decay; the current token gets a bonus instead of the state."""
+
+    STREAMS = "rkvgw"
+
+    def __init__(self, width: int, heads: int, dim: int, lowrank: int, eps: float):
+        super().__init__()
+        self.width, self.heads, self.dim, self.eps = width, heads, dim, eps
+        n = heads * dim
+        self.mu = _f32(5, width)
+        # r, k, v, g share the output size: one batched GEMM over four mixes
+        self.rkvg = nn.Parameter(torch.empty(4, n, width), requires_grad=False)
+        nn.init.normal_(self.rkvg, std=width ** -0.5)
+        self.w1 = Proj(width, lowrank)
+        self.w2 = Proj(lowrank, n)
+        self.w0 = _f32(n)
+        self.u = _f32(heads, dim)
+        self.norm = _f32(n)
+        self.o_proj = Proj(n, width)
+
+    def state_spec(self):
+        return {"prev": (1, self.width), "s": (self.heads, self.dim, self.dim)}
+
+    def kv_spec(self):
+        return None
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        H, D = self.heads, self.dim
+        mixes = sops.token_shift_mix(h, self.mu, state["prev"], fb.seq)
+        rkvg = torch.bmm(mixes[:4], self.rkvg.transpose(1, 2))  # [4, T, n]
+        lr = torch.tanh(self.w1(mixes[4]).float()).to(h.dtype)
+        wpre = self.w2(lr)
+        o = sops.linear_attn_scan(
+            rkvg[0].view(T, H, D), rkvg[1].view(T, H, D), rkvg[2].view(T, H, D),
+            wpre.view(T, H, D), self.u, state["s"], fb.seq, w_bias=self.w0,
+        )
+        y = torch.empty((T, H * D), dtype=h.dtype, device=h.device)
+        sops.gated_rmsnorm(o.view(T, H * D), self.norm, rkvg[3], H, "silu",
+                           self.eps, y)
+        return self.o_proj(y)
+
+
+class ChunkedAttention(nn.Module):
+    """Softmax attention restricted to position-aligned chunks, with grouped
+    key/value heads, separate key and value sizes, short convolutions on the
+    projected q/k/v, rotary on leading interleaved pairs and a tanh cap.
+    Projections are owned by the caller (so they can be fused with a
+    sibling's); this module takes the projected [T, q|k|v] block."""
+
+    def __init__(self, heads, kv_heads, dim, vdim, conv_taps, rot_dims, rot_base,
+                 scale, softcap, chunk, window=0):
+        super().__init__()
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.softcap = float(scale), float(softcap or 0.0)
+        self.chunk, self.window = int(chunk or 0), int(window or 0)
+        self.sizes = (heads * dim, kv_heads * dim, kv_heads * vdim)
+        self.n_in = sum(self.sizes)
+        self.n_out = heads * vdim
+        self.conv = (
+            CausalConvTails(self.n_in, conv_taps, residual=False)
+            if conv_taps and conv_taps > 0 else None
+        )
+        half = int(rot_dims) // 2
+        i = torch.arange(half, dtype=torch.float64)
+        inv = float(rot_base) ** (-2.0 * i / max(int(rot_dims), 1))
+        self.register_buffer("inv_freq", inv.to(torch.float32), persistent=False)
+
+    def state_spec(self):
+        return {"conv": self.conv.state_shape()} if self.conv is not None else {}
+
+    def kv_spec(self):
+        return (self.kv_heads, self.dim, self.vdim)
+
+    def forward(self, qkv, fb, state, kv_cache, out, out_scale=1.0):
+        T = qkv.shape[0]
+        if self.conv is not None:
+            qkv = self.conv(qkv, fb, state["conv"])
+        nq, nk, nv = self.sizes
+        q = qkv[:, :nq].unflatten(-1, (self.heads, self.dim))
+        k = qkv[:, nq : nq + nk].unflatten(-1, (self.kv_heads, self.dim))
+        v = qkv[:, nq + nk :].unflatten(-1, (self.kv_heads, self.vdim))
+        k_cache, v_cache = kv_cache
+        sops.rope_pairs_and_cache(q, k, v, fb.positions, self.inv_freq, k_cache,
+                                  v_cache, fb.slot_mapping)
+        sops.masked_paged_attention(
+            q, k_cache, v_cache, fb.seq, self.scale,
+            out.unflatten(-1, (self.heads, self.vdim)),
+            softcap=self.softcap, chunk=self.chunk, window=self.window,
+            out_scale=out_scale,
+        )
+        return out
+
+
+class LightningAttention(nn.Module):
+    """Linear attention with a constant per-head state decay, silu on q/k/v,
+    an RMS norm over the concatenated heads and a sigmoid output gate.
+    Takes the projected [T, q|k|v|g] block."""
+
+    def __init__(self, heads, dim, vdim, decay, eps):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.eps = heads, dim, vdim, eps
+        self.sizes = (heads * dim, heads * dim, heads * vdim, heads * vdim)
+        self.n_in = sum(self.sizes)
+        self.n_out = heads * vdim
+        self.register_buffer(
+            "decay", torch.tensor(list(decay), dtype=torch.float32), persistent=False
+        )
+        self.norm = _f32(self.n_out)
+
+    def state_spec(self):
+        return {"s": (self.heads, self.dim, self.vdim)}
+
+    def kv_spec(self):
+        return None
+
+    def forward(self, qkvg, fb, state, out, out_scale=1.0):
+        T = qkvg.shape[0]
+        H, D, Dv = self.heads, self.dim, self.vdim
+        a, b, c, _ = self.sizes
+        q = qkvg[:, :a].unflatten(-1, (H, D))
+        k = qkvg[:, a : a + b].unflatten(-1, (H, D))
+        v = qkvg[:, a + b : a + b + c].unflatten(-1, (H, Dv))
+        g = qkvg[:, a + b + c :]
+        o = sops.linear_attn_scan(q, k, v, self.decay, None, state["s"], fb.seq,
+                                  silu_inputs=True)
+        sops.gated_rmsnorm(o.view(T, H * Dv), self.norm, g, 1, "sigmoid",
+                           self.eps, out, out_scale)
+        return out
+
+
+class ParallelMixer(nn.Module):
+    """Chunked softmax attention and lightning attention fed by one input, the
+    same input, summed with fixed scales. Both input projections are one
+    GEMM; both output projections are one GEMM over the concatenated
+    (pre-scaled) branch outputs."""
+
+    def __init__(self, width, left: ChunkedAttention, right: LightningAttention,
+                 left_scale: float, right_scale: float):
+        super().__init__()
+        self.left, self.right = left, right
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+        self.in_proj = Proj(width, left.n_in + right.n_in)
+        self.o_proj = Proj(left.n_out + right.n_out, width)
+
+    def state_spec(self):
+        spec = {"left." + k: v for k, v in self.left.state_spec().items()}
+        spec.update({"right." + k: v for k, v in self.right.state_spec().items()})
+        return spec
+
+    def kv_spec(self):
+        return self.left.kv_spec()
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        proj = self.in_proj(h)
+        nl = self.left.n_in
+        cat = torch.empty((T, self.left.n_out + self.right.n_out), dtype=h.dtype,
+                          device=h.device)
+        ls = {k[5:]: v for k, v in state.items() if k.startswith("left.")}
+        rs = {k[6:]: v for k, v in state.items() if k.startswith("right.")}
+        self.left(proj[:, :nl], fb, ls, kv_cache, cat[:, : self.left.n_out],
+                  self.left_scale)
+        self.right(proj[:, nl:], fb, rs, cat[:, self.left.n_out :],
+                   self.right_scale)
+        return self.o_proj(cat)
+
+
+class SquaredReluMLP(nn.Module):
+    """Dense feed-forward: down(relu(up(h))^2)."""
+
+    def __init__(self, width: int, ff: int):
+        super().__init__()
+        self.up = Proj(width, ff)
+        self.down = Proj(ff, width)
+
+    def forward(self, h):
+        return self.down(sops.relu_squared(self.up(h)))

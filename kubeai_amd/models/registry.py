@@ -1,0 +1,32 @@
+"""Model registry: arch config -> model class. The runner builds whatever the
+checkpoint's config names; a new family registers here."""
+from __future__ import annotations
+
+
+def _llama():
+    from .llama import LlamaForCausalLM
+
+    return LlamaForCausalLM
+
+
+def _dulotar():
+    from .hybrid import DulotarForCausalLM
+
+    return DulotarForCausalLM
+
+
+MODEL_REGISTRY = {
+    "llama": _llama,
+    "mixtral": _llama,
+    "dulotar": _dulotar,
+}
+
+
+def model_class(architecture: str):
+    try:
+        return MODEL_REGISTRY[architecture]()
+    except KeyError:
+        raise ValueError(
+            f"no model class registered for architecture {architecture!r}; "
+            f"known: {sorted(MODEL_REGISTRY)}"
+        ) from None

@@ -1,0 +1,387 @@
+"""Sequence-state ops: recurrences, short convolutions and chunk-masked
+attention over the token-packed batch.
+
+A packed step holds several *runs*: the tokens one sequence contributes
+this step (one token for a decoding sequence, a prompt portion for a
+prefilling one). Everything that carries per-sequence state across steps
+takes a ``SeqMeta`` describing the runs and a state tensor indexed by the
+sequence's *state slot* (engine/statecache.py). Conventions:
+
+  - state tensors are fp32, ``[num_slots, ...]``; a run with slot -1 (bucket
+    padding) reads zeros and writes nothing;
+  - a run whose first token sits at position 0 starts from zero state
+    whatever the slot holds, so a slot can be handed to a new sequence
+    without clearing it;
+  - activations are bf16 or fp32 (the serving dtype); recurrences, decays,
+    gates of a recurrence, norms and attention scores are fp32 inside.
+
+Dispatch follows kubeai_amd.ops: CPU tensors run the torch references below
+(also the numerics contract of the kernels); GPU tensors require the
+``kubeai_amd._C_seq`` HIP extension and fail loudly without it.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Optional
+
+import torch
+
+_C = None
+_C_IMPORT_ERROR: Exception | None = None
+try:
+    from kubeai_amd import _C_seq as _C  # type: ignore[attr-defined,no-redef]
+except Exception as e:  # pragma: no cover
+    _C_IMPORT_ERROR = e
+
+
+def have_seq_ext() -> bool:
+    return _C is not None
+
+
+def _require_ext() -> None:
+    if _C is None:
+        raise RuntimeError(
+            "kubeai_amd._C_seq (sequence-state HIP kernels) is not built but a "
+            "GPU tensor reached the ops layer. Build it with "
+            "`KUBEAI_BUILD_ONLY=_C_seq python setup.py build_ext --inplace`. "
+            f"Original import error: {_C_IMPORT_ERROR!r}"
+        )
+
+
+@dataclasses.dataclass
+class SeqMeta:
+    """Runs of the packed token stream, in packing order."""
+
+    start_loc: torch.Tensor   # int32 [n_seq + 1] offsets into the stream
+    slots: torch.Tensor       # int32 [n_seq] state slot, -1 = none
+    token_seq: torch.Tensor   # int32 [T] run index of every token
+    positions: torch.Tensor   # int32 [T] position of every token in its sequence
+    block_tables: Optional[torch.Tensor]  # int32 [n_seq, max_blocks]
+    n_seq: int
+    max_len: int              # longest run (host value, sizes grids)
+
+    def runs(self):
+        """(start, length, slot, first position) per run — host values, for
+        the CPU references only."""
+        sl = self.start_loc.tolist()
+        slots = self.slots.tolist()
+        pos = self.positions
+        for i in range(self.n_seq):
+            s0, n = sl[i], sl[i + 1] - sl[i]
+            if n > 0:
+                yield s0, n, slots[i], int(pos[s0])
+
+    @staticmethod
+    def build(runs, positions, device, block_tables=None) -> "SeqMeta":
+        """runs: list of (length, slot). positions: int32 tensor [T]."""
+        import numpy as np
+
+        lens = np.asarray([r[0] for r in runs], dtype=np.int64)
+        start = np.zeros(len(runs) + 1, dtype=np.int32)
+        np.cumsum(lens, out=start[1:])
+        tok = np.repeat(np.arange(len(runs), dtype=np.int32), lens)
+        return SeqMeta(
+            start_loc=torch.from_numpy(start).to(device),
+            slots=torch.tensor([r[1] for r in runs], dtype=torch.int32, device=device),
+            token_seq=torch.from_numpy(tok).to(device),
+            positions=positions,
+            block_tables=block_tables,
+            n_seq=len(runs),
+            max_len=int(lens.max()) if len(runs) else 0,
+        )
+
+
+# ---------------------------------------------------------------------------
+# norms
+# ---------------------------------------------------------------------------
+
+def add_layernorm(branch, residual, weight, bias, eps: float, out_dtype):
+    """residual (fp32, in place) += branch; returns LayerNorm(residual) * w + b
+    in ``out_dtype``. The variance is the mean squared deviation. branch may
+    be None (first norm of the model)."""
+    if residual.is_cuda:
+        _require_ext()
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        _C.add_layernorm(out, branch, residual, weight, bias, eps)
+        return out
+    if branch is not None:
+        residual.add_(branch.float())
+    mu = residual.mean(-1, keepdim=True)
+    d = residual - mu
+    var = (d * d).mean(-1, keepdim=True)
+    return (d * torch.rsqrt(var + eps) * weight + bias).to(out_dtype)
+
+
+def gated_rmsnorm(o, weight, gate, groups: int, gate_act: str, eps: float,
+                  out, out_scale: float = 1.0):
+    """out = o / rms(o over each of `groups` equal slices) * weight
+    * act(gate) * out_scale. o is fp32 [T, C]; gate [T, C] may be a strided
+    column view; out [T, C] may be a strided column view of a wider buffer.
+    gate_act: "none" (gate already activated), "sigmoid" or "silu"."""
+    if o.is_cuda:
+        _require_ext()
+        _C.gated_rmsnorm(out, o, weight, gate, groups,
+                         {"none": 0, "sigmoid": 1, "silu": 2}[gate_act], eps,
+                         out_scale)
+        return out
+    T, C = o.shape
+    og = o.view(T, groups, C // groups)
+    n = og * torch.rsqrt((og * og).mean(-1, keepdim=True) + eps)
+    g = gate.float()
+    if gate_act == "sigmoid":
+        g = torch.sigmoid(g)
+    elif gate_act == "silu":
+        g = g * torch.sigmoid(g)
+    out.copy_((n.reshape(T, C) * weight * g * out_scale).to(out.dtype))
+    return out
+
+
+def relu_squared(x):
+    """relu(x)^2, elementwise (fp32 inside)."""
+    if x.is_cuda:
+        _require_ext()
+        out = torch.empty_like(x)
+        _C.relu_squared(out, x)
+        return out
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# short causal convolutions with carried tails
+# ---------------------------------------------------------------------------
+
+def causal_conv(x, w, tails, meta: SeqMeta, residual: bool):
+    """Depthwise causal convolution over time inside every run.
+
+    x [T, C] (row-strided view allowed); w fp32 [C, taps]:
+    y_t = sum_j w[:, j] * x_(t - taps + 1 + j)  (+ x_t if residual).
+    tails fp32 [slots, taps-1, C] holds each sequence's last taps-1 inputs
+    (row i = input at position P - (taps-1) + i, P = the next position) and
+    is advanced past this step's tokens. Inputs before position 0 are zero.
+    """
+    taps = w.shape[1]
+    if x.is_cuda:
+        _require_ext()
+        y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _C.causal_conv(y, x, w, tails, meta.start_loc, meta.slots,
+                       meta.token_seq, meta.positions, residual)
+        return y
+    y = torch.empty(x.shape, dtype=x.dtype)
+    C = x.shape[1]
+    for s0, n, slot, p0 in meta.runs():
+        xs = x[s0 : s0 + n].float()
+        hist = torch.zeros(taps - 1, C)
+        if slot >= 0:
+            hist = tails[slot].clone()
+            for i in range(taps - 1):
+                if p0 - (taps - 1) + i < 0:
+                    hist[i] = 0
+        full = torch.cat([hist, xs])
+        acc = xs.clone() if residual else torch.zeros_like(xs)
+        for j in range(taps):
+            acc += w[:, j] * full[j : j + n]
+        y[s0 : s0 + n] = acc.to(x.dtype)
+        if slot >= 0:
+            tails[slot] = full[n : n + taps - 1]
+    return y
+
+
+def token_shift_mix(h, mu, prev, meta: SeqMeta):
+    """mixes[s] = h + (h' - h) * mu[s], h' the previous token's h (zeros at
+    position 0; across steps it comes from prev fp32 [slots, 1, C], which is
+    advanced). h [T, C], mu fp32 [S, C] -> [S, T, C]."""
+    if h.is_cuda:
+        _require_ext()
+        out = torch.empty((mu.shape[0],) + tuple(h.shape), dtype=h.dtype,
+                          device=h.device)
+        _C.token_shift_mix(out, h, mu, prev, meta.start_loc, meta.slots,
+                           meta.token_seq, meta.positions)
+        return out
+    out = torch.empty((mu.shape[0],) + tuple(h.shape), dtype=h.dtype)
+    for s0, n, slot, p0 in meta.runs():
+        hs = h[s0 : s0 + n].float()
+        first = torch.zeros(1, h.shape[1])
+        if slot >= 0 and p0 > 0:
+            first = prev[slot].clone()
+        hp = torch.cat([first, hs[:-1]])
+        out[:, s0 : s0 + n] = (hs + (hp - hs) * mu.unsqueeze(1)).to(h.dtype)
+        if slot >= 0:
+            prev[slot] = hs[-1:]
+    return out
+
+
+# ---------------------------------------------------------------------------
+# recurrences
+# ---------------------------------------------------------------------------
+
+def mingru_scan(zxg, bz, bx, state, meta: SeqMeta):
+    """Elementwise gated recurrence over packed projections zxg [T, 3n]
+    (z | x | g): z = sigmoid(z + bz), u = x + bx,
+    c = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),
+    S_t = (1 - z) S_(t-1) + z c, y_t = S_t * silu(g). state fp32 [slots, n]."""
+    n = bz.numel()
+    if zxg.is_cuda:
+        _require_ext()
+        y = torch.empty((zxg.shape[0], n), dtype=zxg.dtype, device=zxg.device)
+        _C.mingru_scan(y, zxg, bz, bx, state, meta.start_loc, meta.slots,
+                       meta.positions)
+        return y
+    y = torch.empty((zxg.shape[0], n), dtype=zxg.dtype)
+    for s0, ln, slot, p0 in meta.runs():
+        blk = zxg[s0 : s0 + ln].float()
+        z = torch.sigmoid(blk[:, :n] + bz)
+        u = blk[:, n : 2 * n] + bx
+        g = blk[:, 2 * n :]
+        c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        S = state[slot].clone() if (slot >= 0 and p0 > 0) else torch.zeros(n)
+        for t in range(ln):
+            S = (1 - z[t]) * S + z[t] * c[t]
+            y[s0 + t] = (S * (g[t] * torch.sigmoid(g[t]))).to(zxg.dtype)
+        if slot >= 0:
+            state[slot] = S
+    return y
+
+
+def linear_attn_scan(q, k, v, decay, bonus, state, meta: SeqMeta, *,
+                     w_bias=None, silu_inputs: bool = False):
+    """Matrix-state linear attention, per head S [D, Dv] (fp32).
+
+    Two forms share the kernel:
+      * per-token channel decay (decay [T, H, D] holds pre-activations,
+        w = exp(-exp(decay + w_bias))) with a bonus u [H, D] for the current
+        token: o_t = (S + diag(u) k v^T)^T q, then S <- diag(w) S + k v^T;
+      * constant per-head decay (decay fp32 [H], bonus None):
+        S <- decay S + k v^T, then o_t = S^T q.
+    silu_inputs applies silu to q, k, v first. q, k [T, H, D], v [T, H, Dv]
+    (strided views allowed); returns o fp32 [T, H, Dv].
+    """
+    T, H, D = q.shape
+    Dv = v.shape[2]
+    per_token = decay.dim() == 3
+    if q.is_cuda:
+        _require_ext()
+        o = torch.empty((T, H, Dv), dtype=torch.float32, device=q.device)
+        _C.linear_attn_scan(o, q, k, v, decay, bonus, w_bias, state,
+                            meta.start_loc, meta.slots, meta.positions,
+                            silu_inputs)
+        return o
+    o = torch.empty((T, H, Dv), dtype=torch.float32)
+    act = (lambda a: a * torch.sigmoid(a)) if silu_inputs else (lambda a: a)
+    for s0, n, slot, p0 in meta.runs():
+        qs, ks, vs = (act(a[s0 : s0 + n].float()) for a in (q, k, v))
+        if per_token:
+            w = torch.exp(-torch.exp(decay[s0 : s0 + n].float() + w_bias.view(H, D)))
+        S = (state[slot].clone() if (slot >= 0 and p0 > 0)
+             else torch.zeros(H, D, Dv))
+        for t in range(n):
+            kv = ks[t].unsqueeze(-1) * vs[t].unsqueeze(-2)
+            if per_token:
+                o[s0 + t] = torch.einsum(
+                    "hkv,hk->hv", S + bonus.unsqueeze(-1) * kv, qs[t])
+                S = w[t].unsqueeze(-1) * S + kv
+            else:
+                S = decay.view(H, 1, 1) * S + kv
+                o[s0 + t] = torch.einsum("hkv,hk->hv", S, qs[t])
+        if slot >= 0:
+            state[slot] = S
+    return o
+
+
+# ---------------------------------------------------------------------------
+# rotary (interleaved pairs, leading dims) + paged cache write
+# ---------------------------------------------------------------------------
+
+def rope_pairs_and_cache(q, k, v, positions, inv_freq, k_cache, v_cache,
+                         slot_mapping):
+    """Rotate adjacent pairs (2i, 2i+1) of the first 2*len(inv_freq) dims of
+    every q and k head by angle position * inv_freq[i] (fp32 angles); q is
+    rotated in place, rotated k and v go to the paged caches
+    (k_cache [blocks, G, block, D], v_cache [blocks, G, block, Dv]) at
+    slot_mapping (slot < 0: no write). q [T, H, D], k [T, G, D],
+    v [T, G, Dv] may be strided views."""
+    if q.is_cuda:
+        _require_ext()
+        _C.rope_pairs_and_cache(q, k, v, positions, inv_freq, k_cache, v_cache,
+                                slot_mapping)
+        return q
+    half = inv_freq.numel()
+    a = positions.float().unsqueeze(-1) * inv_freq  # [T, half]
+    c, s = torch.cos(a).unsqueeze(1), torch.sin(a).unsqueeze(1)
+
+    def rot(x):
+        xf = x.float()
+        u = xf[..., 0 : 2 * half : 2]
+        w = xf[..., 1 : 2 * half : 2]
+        out = xf.clone()
+        out[..., 0 : 2 * half : 2] = u * c - w * s
+        out[..., 1 : 2 * half : 2] = w * c + u * s
+        return out.to(x.dtype)
+
+    q.copy_(rot(q))
+    kr = rot(k)
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    blk = (slot_mapping[ok] // bs).long()
+    off = (slot_mapping[ok] % bs).long()
+    k_cache[blk, :, off] = kr[ok].to(k_cache.dtype)
+    v_cache[blk, :, off] = v[ok].to(v_cache.dtype)
+    return q
+
+
+# ---------------------------------------------------------------------------
+# masked paged attention (decode tokens and prompt portions alike)
+# ---------------------------------------------------------------------------
+
+def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
+                           out, *, softcap: float = 0.0, chunk: int = 0,
+                           window: int = 0, out_scale: float = 1.0):
+    """Softmax attention of every packed token over its own sequence's cached
+    keys. The token at position i sees j <= i with, when chunk > 0,
+    floor(j / chunk) == floor(i / chunk) (position-aligned chunks) and, when
+    window > 0, j > i - window. Scores are (q . k) * scale, then
+    softcap * tanh(score / softcap) if softcap > 0; all in fp32.
+    q [T, H, D] (strided ok), caches [blocks, G, block, D | Dv];
+    out [T, H, Dv] may be a strided view; out = attention * out_scale."""
+    if q.is_cuda:
+        _require_ext()
+        _C.masked_paged_attention(out, q, k_cache, v_cache, meta.block_tables,
+                                  meta.token_seq, meta.positions, scale,
+                                  softcap, chunk, window, out_scale)
+        return out
+    T, H, D = q.shape
+    G, bs = k_cache.shape[1], k_cache.shape[2]
+    rep = H // G
+    bt = meta.block_tables
+    sl = meta.start_loc.tolist()
+    for si in range(meta.n_seq):
+        s0, n = sl[si], sl[si + 1] - sl[si]
+        if n == 0:
+            continue
+        pos = meta.positions[s0 : s0 + n].long()
+        L = int(pos.max()) + 1
+        lo = 0
+        if chunk > 0:
+            lo = (int(pos.min()) // chunk) * chunk
+        if window > 0:
+            lo = max(lo, int(pos.min()) - window + 1)
+        j = torch.arange(lo, L)
+        blk = bt[si][(j // bs)].long()
+        ks = k_cache[blk, :, j % bs].float()  # [L', G, D]
+        vs = v_cache[blk, :, j % bs].float()
+        ks = ks.repeat_interleave(rep, dim=1)
+        vs = vs.repeat_interleave(rep, dim=1)
+        s = torch.einsum("thd,lhd->htl", q[s0 : s0 + n].float(), ks) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        vis = j.view(1, -1) <= pos.view(-1, 1)
+        if chunk > 0:
+            vis &= (j.view(1, -1) // chunk) == (pos.view(-1, 1) // chunk)
+        if window > 0:
+            vis &= j.view(1, -1) > pos.view(-1, 1) - window
+        s = s.masked_fill(~vis.unsqueeze(0), float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        o = torch.einsum("htl,lhd->thd", p, vs) * out_scale
+        out[s0 : s0 + n] = o.to(out.dtype)
+    return out
