@@ -30,3 +30,15 @@ def model_class(architecture: str):
             f"no model class registered for architecture {architecture!r}; "
             f"known: {sorted(MODEL_REGISTRY)}"
         ) from None
+
+
+# HIP extensions (kubeai_amd.<name>) whose kernels a family's forward uses
+MODEL_EXTENSIONS = {
+    "llama": ("_C",),
+    "mixtral": ("_C",),
+    "dulotar": ("_C_seq",),
+}
+
+
+def required_extensions(architecture: str) -> tuple:
+    return MODEL_EXTENSIONS.get(architecture, ("_C",))

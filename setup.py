@@ -16,49 +16,69 @@ os.environ.setdefault("PYTORCH_ROCM_ARCH", "gfx950")
 from torch.utils import cpp_extension  # noqa: E402
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(ROOT, "kubeai_amd", "csrc")
 
-sources = sorted(
-    glob.glob(os.path.join(CSRC, "*.cpp")) + glob.glob(os.path.join(CSRC, "*.hip"))
-)
+# extension name -> source folder. KUBEAI_BUILD_ONLY=<name>[,<name>] builds a
+# subset (a model family's first start compiles only what it needs).
+EXTENSIONS = {
+    "_C": os.path.join(ROOT, "kubeai_amd", "csrc"),
+    "_C_seq": os.path.join(ROOT, "kubeai_amd", "csrc_seq"),
+}
+_only = [n for n in os.environ.get("KUBEAI_BUILD_ONLY", "").split(",") if n]
+for _n in _only:
+    if _n not in EXTENSIONS:
+        raise SystemExit(f"unknown extension {_n!r}; known: {sorted(EXTENSIONS)}")
 
-# torch's hipify/ninja pipeline tracks no header dependencies for .hip
-# objects: a common.h edit would silently ship stale kernels. Touch every
-# .hip newer than its headers so the pipeline rebuilds them.
-_hdr_mtime = max(
-    (os.path.getmtime(h) for h in glob.glob(os.path.join(CSRC, "*.h"))),
-    default=0.0,
-)
-for _src in list(sources):
-    if (
-        _src.endswith(".hip")
-        and not _src.endswith("_hip.hip")
-        and os.path.exists(_src)
-        and os.path.getmtime(_src) < _hdr_mtime
-    ):
-        os.utime(_src, None)
-        _gen = _src[:-4] + "_hip.hip"
-        if os.path.exists(_gen):
-            os.remove(_gen)
-            sources = [s for s in sources if s != _gen]
-# drop hipify artifacts whose base source was deleted or touched
-sources = [s for s in sources if os.path.exists(s)]
+
+def _sources(csrc: str) -> list:
+    sources = sorted(
+        glob.glob(os.path.join(csrc, "*.cpp")) + glob.glob(os.path.join(csrc, "*.hip"))
+    )
+    # torch's hipify/ninja pipeline tracks no header dependencies for .hip
+    # objects: a header edit would silently ship stale kernels. Touch every
+    # .hip older than its headers so the pipeline rebuilds them.
+    hdr_mtime = max(
+        (
+            os.path.getmtime(h)
+            for h in glob.glob(os.path.join(csrc, "*.h"))
+            if not h.endswith("_hip.h")
+        ),
+        default=0.0,
+    )
+    for src in list(sources):
+        if (
+            src.endswith(".hip")
+            and not src.endswith("_hip.hip")
+            and os.path.exists(src)
+            and os.path.getmtime(src) < hdr_mtime
+        ):
+            os.utime(src, None)
+            gen = src[:-4] + "_hip.hip"
+            if os.path.exists(gen):
+                os.remove(gen)
+                sources = [s for s in sources if s != gen]
+    # drop hipify artifacts: they are regenerated from their base source
+    return [s for s in sources if os.path.exists(s) and not s.endswith("_hip.hip")]
+
 
 setup(
     name="kubeai_amd_C",
     ext_modules=[
         cpp_extension.CUDAExtension(
-            name="kubeai_amd._C",
-            sources=sources,
+            name="kubeai_amd." + name,
+            sources=_sources(csrc),
             extra_compile_args={
                 "cxx": ["-O3", "-std=c++17"],
                 "nvcc": [
                     "-O3",
                     "-std=c++17",
                     "--offload-arch=gfx950",
+                    # packed fp32 math is left to scalar instructions
+                    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                 ],
             },
         )
+        for name, csrc in EXTENSIONS.items()
+        if not _only or name in _only
     ],
     cmdclass={"build_ext": cpp_extension.BuildExtension},
 )
