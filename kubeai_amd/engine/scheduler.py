@@ -102,6 +102,7 @@ class Request:
         # slot of the per-sequence recurrent state (models that carry one);
         # -1 while not admitted
         self.state_slot: int = -1
+        self.recompute_len = 0  # set by preemption, see prefill_len
         self.block_hashes: list[int] = []  # sealed-block hash chain
         self.num_cached_prompt_tokens = 0  # prefix-cache hits at admission
 
@@ -111,8 +112,15 @@ class Request:
         return len(self.tokens) - self.num_prompt_tokens
 
     @property
+    def prefill_len(self) -> int:
+        """Tokens to run as prompt portions before the next token is sampled:
+        the prompt, or after a preemption everything the sequence holds (its
+        generated tokens are recomputed with the prompt)."""
+        return max(self.num_prompt_tokens, self.recompute_len)
+
+    @property
     def in_prefill(self) -> bool:
-        return self.num_computed < self.num_prompt_tokens
+        return self.num_computed < self.prefill_len
 
     @property
     def output_token_ids(self) -> list[int]:
@@ -128,7 +136,7 @@ class ScheduledSeq:
     @property
     def samples(self) -> bool:
         """Does this step produce a sampled token for the request?"""
-        return self.chunk_start + self.chunk_len >= self.req.num_prompt_tokens
+        return self.chunk_start + self.chunk_len >= self.req.prefill_len
 
 
 @dataclasses.dataclass
@@ -263,7 +271,7 @@ class Scheduler:
         for req in [r for r in list(self.running) if r.in_prefill]:
             if budget <= 0 or req.status != RequestStatus.RUNNING or defer_prefill:
                 continue
-            chunk = min(req.num_prompt_tokens - req.num_computed, budget)
+            chunk = min(req.prefill_len - req.num_computed, budget)
             if not self._ensure_blocks(req, req.num_computed + chunk, preempted):
                 continue  # req itself got preempted
             prefill.append(ScheduledSeq(req, req.num_computed, chunk))
@@ -278,7 +286,7 @@ class Scheduler:
             and len(self.running) < self.max_num_seqs
         ):
             req = self.waiting[0]
-            n_prompt = req.num_prompt_tokens
+            n_prompt = req.prefill_len
             if self.sm is not None and self.sm.num_free == 0:
                 break
             try:
@@ -360,6 +368,7 @@ class Scheduler:
     def _preempt(self, req: Request, preempted: list[Request]) -> None:
         self._release(req)
         req.block_hashes = []
+        req.recompute_len = len(req.tokens)
         req.num_computed = 0
         req.status = RequestStatus.WAITING
         self.running.remove(req)

@@ -94,6 +94,22 @@ def rotate_interleaved(x, pos, base, dims):
     return x
 
 
+def chunk_softmax(q, k, v, scale, cap, size):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv] -> [T, H, Dv]; position t sees
+    j <= t with floor(j / size) == floor(t / size)."""
+    T, H, _ = q.shape
+    G, Dv = k.shape[1], v.shape[2]
+    out = torch.zeros(T, H, Dv, dtype=q.dtype)
+    for t in range(T):
+        lo = (t // size) * size
+        for hd in range(H):
+            g = hd // (H // G)
+            s = (k[lo : t + 1, g] @ q[t, hd]) * scale
+            s = cap * torch.tanh(s / cap)
+            out[t, hd] = torch.softmax(s, 0) @ v[lo : t + 1, g]
+    return out
+
+
 def chunked_attention(h, W, p, m):
     """Softmax attention inside position-aligned chunks, with short
     convolutions on q/k/v, partial rotary and a tanh cap on the scores."""
@@ -105,15 +121,7 @@ def chunked_attention(h, W, p, m):
     pos = torch.arange(T)
     q = rotate_interleaved(q, pos, m["rot"]["base"], m["rot"]["dims"])
     k = rotate_interleaved(k, pos, m["rot"]["base"], m["rot"]["dims"])
-    cap, size = m["softcap"], m["mask"]["size"]
-    out = torch.zeros(T, H, Dv, dtype=h.dtype)
-    for t in range(T):
-        lo = (t // size) * size
-        for hd in range(H):
-            g = hd // (H // G)
-            s = (k[lo : t + 1, g] @ q[t, hd]) * m["scale"]
-            s = cap * torch.tanh(s / cap)
-            out[t, hd] = torch.softmax(s, 0) @ v[lo : t + 1, g]
+    out = chunk_softmax(q, k, v, m["scale"], m["softcap"], m["mask"]["size"])
     return out.reshape(T, H * Dv) @ W[p + "o"].T
 
 
