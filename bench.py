@@ -89,6 +89,11 @@ def get_args():
         "= fp8 for the Llama configs (the reference headline model is "
         "Llama-3.1-8B-Instruct-FP8, i.e. fp8 IS the named precision).",
     )
+    p.add_argument("--compare-hybrid", action="store_true",
+                   help="instead of the headline workload: prefill/decode "
+                   "throughput of the Dulotar hybrid beside an equal-size Llama "
+                   "(benchmarks/hybrid_compare.py)")
+    p.add_argument("--compare-sizes", default="1k,2k,4k")
     return p.parse_args()
 
 
@@ -144,6 +149,11 @@ class VirtualUser:
 
 def main():
     args = get_args()
+    if args.compare_hybrid:
+        from benchmarks import hybrid_compare
+
+        hybrid_compare.main(args)
+        return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", str(rank)))

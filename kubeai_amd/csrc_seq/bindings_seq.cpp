@@ -18,7 +18,7 @@ void token_shift_mix(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
                      torch::Tensor positions);
 void mingru_scan(torch::Tensor y, torch::Tensor zxg, torch::Tensor bz,
                  torch::Tensor bx, torch::Tensor state, torch::Tensor start_loc,
-                 torch::Tensor slots, torch::Tensor positions);
+                 torch::Tensor slots, torch::Tensor positions, int64_t max_len);
 void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                       torch::Tensor v, torch::Tensor decay,
                       c10::optional<torch::Tensor> bonus,

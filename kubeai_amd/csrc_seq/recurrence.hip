@@ -7,30 +7,71 @@
 
 namespace {
 
-// grid (n_seq, ceil(n / 256)): one thread walks one channel of one run.
+constexpr int kGruSeg = 64;  // tokens per segment of a run
+
+// The recurrence S_t = a_t S_(t-1) + b_t composes: a segment of a run maps
+// its incoming state S to A S + B. Long runs are cut into segments of
+// kGruSeg tokens that are walked in parallel.
+//
+// Pass 1, grid (n_seq, n_segments, ceil(n / 256)), only when a run spans
+// more than one segment: (A, B) of every segment.
+template <typename T>
+__global__ void mingru_segments_kernel(
+    float* __restrict__ segA, float* __restrict__ segB,
+    const T* __restrict__ zxg, const float* __restrict__ bz,
+    const float* __restrict__ bx, const int* __restrict__ start_loc, int n,
+    int nseg) {
+  const int s = blockIdx.x, g = blockIdx.y;
+  const int c = blockIdx.z * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  const int s0 = start_loc[s], s1 = start_loc[s + 1];
+  const int t0 = s0 + g * kGruSeg, t1 = min(t0 + kGruSeg, s1);
+  if (t0 >= s1) return;
+  const float bzc = bz[c], bxc = bx[c];
+  float A = 1.f, B = 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const T* row = zxg + (size_t)t * 3 * n;
+    const float z = sigmoid_f(ldf(row + c) + bzc);
+    const float u = ldf(row + n + c) + bxc;
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+    A *= 1.0f - z;
+    B = (1.0f - z) * B + z * cand;
+  }
+  segA[((size_t)s * nseg + g) * n + c] = A;
+  segB[((size_t)s * nseg + g) * n + c] = B;
+}
+
+// Pass 2, same grid: fold the earlier segments into the incoming state,
+// then walk the own segment and write y; the last segment stores the state.
 template <typename T>
 __global__ void mingru_scan_kernel(
     T* __restrict__ y, const T* __restrict__ zxg, const float* __restrict__ bz,
     const float* __restrict__ bx, float* __restrict__ state,
+    const float* __restrict__ segA, const float* __restrict__ segB,
     const int* __restrict__ start_loc, const int* __restrict__ slots,
-    const int* __restrict__ positions, int n) {
-  const int s = blockIdx.x;
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    const int* __restrict__ positions, int n, int nseg) {
+  const int s = blockIdx.x, g = blockIdx.y;
+  const int c = blockIdx.z * blockDim.x + threadIdx.x;
   if (c >= n) return;
   const int s0 = start_loc[s], s1 = start_loc[s + 1], slot = slots[s];
-  if (s1 <= s0) return;
+  const int t0 = s0 + g * kGruSeg, t1 = min(t0 + kGruSeg, s1);
+  if (t0 >= s1) return;
   float S = (slot >= 0 && positions[s0] > 0) ? state[(size_t)slot * n + c] : 0.f;
+  for (int gg = 0; gg < g; ++gg) {
+    const size_t i = ((size_t)s * nseg + gg) * n + c;
+    S = segA[i] * S + segB[i];
+  }
   const float bzc = bz[c], bxc = bx[c];
-  for (int t = s0; t < s1; ++t) {
+  for (int t = t0; t < t1; ++t) {
     const T* row = zxg + (size_t)t * 3 * n;
     const float z = sigmoid_f(ldf(row + c) + bzc);
     const float u = ldf(row + n + c) + bxc;
-    const float g = ldf(row + 2 * n + c);
+    const float gt = ldf(row + 2 * n + c);
     const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
     S = (1.0f - z) * S + z * cand;
-    stf(y + (size_t)t * n + c, S * silu_f(g));
+    stf(y + (size_t)t * n + c, S * silu_f(gt));
   }
-  if (slot >= 0) state[(size_t)slot * n + c] = S;
+  if (slot >= 0 && t1 == s1) state[(size_t)slot * n + c] = S;
 }
 
 constexpr int kScanTile = 16;  // tokens staged per barrier
@@ -116,11 +157,110 @@ __global__ void linear_attn_scan_kernel(
     for (int i = tid; i < D * Dv; i += nthr) sp[i] = S[i];
 }
 
+// Register-state form for key sizes D = 16 * kQ (<= 128). grid
+// (n_seq * H * ceil(Dv / 16)), one wave per block: the wave owns 16 value
+// columns of one head; lane (r, c) keeps rows [r D/4, (r+1) D/4) of column c
+// in registers, so a token costs D/4 fused steps per lane and two shuffles
+// to join the four partial outputs. q/k/decay of kScanTile tokens are staged
+// through LDS with activations and decays applied once per element.
+template <typename T, bool kPerToken, int kQ>
+__global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
+    float* __restrict__ o, const T* __restrict__ q, int64_t q_stride,
+    const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
+    int64_t v_stride, const T* __restrict__ decay_pre, int64_t d_stride,
+    const float* __restrict__ decay_const, const float* __restrict__ bonus,
+    const float* __restrict__ w_bias, float* __restrict__ state,
+    const int* __restrict__ start_loc, const int* __restrict__ slots,
+    const int* __restrict__ positions, int H, int Dv, int ncb,
+    int silu_inputs) {
+  constexpr int R = 4 * kQ, D = 4 * R;
+  const int cb = blockIdx.x % ncb;
+  const int h = (blockIdx.x / ncb) % H;
+  const int s = blockIdx.x / (ncb * H);
+  const int s0 = start_loc[s], s1 = start_loc[s + 1], slot = slots[s];
+  if (s1 <= s0) return;
+  __shared__ __attribute__((aligned(16))) float qs[kScanTile * D];
+  __shared__ __attribute__((aligned(16))) float ks[kScanTile * D];
+  __shared__ __attribute__((aligned(16))) float ws[kPerToken ? kScanTile * D : 4];
+  __shared__ float vs[kScanTile * 16];
+  const int lane = threadIdx.x, r = lane >> 4, c = lane & 15;
+  const int j = cb * 16 + c;
+  const bool valid = j < Dv;
+  const bool carry = slot >= 0 && positions[s0] > 0;
+  float* sp = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * D * Dv;
+  float S[R], U[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    S[i] = (carry && valid) ? sp[(size_t)(r * R + i) * Dv + j] : 0.f;
+    U[i] = kPerToken ? bonus[h * D + r * R + i] : 0.f;
+  }
+  const float dc = kPerToken ? 0.f : decay_const[h];
+  for (int t0 = s0; t0 < s1; t0 += kScanTile) {
+    const int nt = min(kScanTile, s1 - t0);
+    __syncthreads();
+    for (int i = lane; i < nt * D; i += WAVE) {
+      const int tt = i / D, d = i % D;
+      float qv = ldf(q + (size_t)(t0 + tt) * q_stride + h * D + d);
+      float kv = ldf(k + (size_t)(t0 + tt) * k_stride + h * D + d);
+      if (silu_inputs) { qv = silu_f(qv); kv = silu_f(kv); }
+      qs[i] = qv;
+      ks[i] = kv;
+      if (kPerToken)
+        ws[i] = expf(-expf(ldf(decay_pre + (size_t)(t0 + tt) * d_stride + h * D + d) +
+                           w_bias[h * D + d]));
+    }
+    for (int i = lane; i < nt * 16; i += WAVE) {
+      const int tt = i / 16, cc = cb * 16 + (i % 16);
+      float vv = cc < Dv ? ldf(v + (size_t)(t0 + tt) * v_stride + h * Dv + cc) : 0.f;
+      if (silu_inputs) vv = silu_f(vv);
+      vs[i] = vv;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vj = vs[tt * 16 + c];
+      const float4* q4 = (const float4*)(qs + tt * D + r * R);
+      const float4* k4 = (const float4*)(ks + tt * D + r * R);
+      const float4* w4 = (const float4*)(ws + (kPerToken ? tt * D + r * R : 0));
+      float acc = 0.f;
+#pragma unroll
+      for (int b = 0; b < kQ; ++b) {
+        const float4 qq = q4[b], kk = k4[b];
+        const float qa[4] = {qq.x, qq.y, qq.z, qq.w};
+        const float ka[4] = {kk.x, kk.y, kk.z, kk.w};
+        float wa[4] = {0.f, 0.f, 0.f, 0.f};
+        if (kPerToken) {
+          const float4 ww = w4[b];
+          wa[0] = ww.x; wa[1] = ww.y; wa[2] = ww.z; wa[3] = ww.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = b * 4 + e;
+          const float kv = ka[e] * vj;
+          if (kPerToken) {
+            acc += qa[e] * (S[i] + U[i] * kv);
+            S[i] = wa[e] * S[i] + kv;
+          } else {
+            S[i] = dc * S[i] + kv;
+            acc += qa[e] * S[i];
+          }
+        }
+      }
+      acc += __shfl_xor(acc, 16, WAVE);
+      acc += __shfl_xor(acc, 32, WAVE);
+      if (r == 0 && valid) o[((size_t)(t0 + tt) * H + h) * Dv + j] = acc;
+    }
+  }
+  if (slot >= 0 && valid) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) sp[(size_t)(r * R + i) * Dv + j] = S[i];
+  }
+}
+
 }  // namespace
 
 void mingru_scan(torch::Tensor y, torch::Tensor zxg, torch::Tensor bz,
                  torch::Tensor bx, torch::Tensor state, torch::Tensor start_loc,
-                 torch::Tensor slots, torch::Tensor positions) {
+                 torch::Tensor slots, torch::Tensor positions, int64_t max_len) {
   check_f32(bz, "bz");
   check_f32(bx, "bx");
   check_f32(state, "state");
@@ -136,16 +276,39 @@ void mingru_scan(torch::Tensor y, torch::Tensor zxg, torch::Tensor bz,
               positions.numel() == zxg.size(0));
   const int n_seq = slots.numel();
   if (n_seq == 0 || zxg.size(0) == 0) return;
+  const int nseg = std::max<int>(1, (max_len + kGruSeg - 1) / kGruSeg);
+  TORCH_CHECK(nseg <= 65535 && (n + 255) / 256 <= 65535);
+  torch::Tensor seg;
+  float* segA = nullptr;
+  float* segB = nullptr;
+  if (nseg > 1) {
+    seg = torch::empty({2, n_seq, nseg, n}, state.options());
+    segA = (float*)seg.data_ptr();
+    segB = segA + (size_t)n_seq * nseg * n;
+  }
+  const dim3 grid(n_seq, nseg, (n + 255) / 256);
   SEQ_DISPATCH_ACT(zxg, {
-    hipLaunchKernelGGL((mingru_scan_kernel<act_t>), dim3(n_seq, (n + 255) / 256),
-                       dim3(256), 0, SEQ_STREAM(), (act_t*)y.data_ptr(),
+    if (nseg > 1)
+      hipLaunchKernelGGL((mingru_segments_kernel<act_t>), grid, dim3(256), 0,
+                         SEQ_STREAM(), segA, segB, (const act_t*)zxg.data_ptr(),
+                         (const float*)bz.data_ptr(), (const float*)bx.data_ptr(),
+                         (const int*)start_loc.data_ptr(), n, nseg);
+    hipLaunchKernelGGL((mingru_scan_kernel<act_t>), grid, dim3(256), 0,
+                       SEQ_STREAM(), (act_t*)y.data_ptr(),
                        (const act_t*)zxg.data_ptr(), (const float*)bz.data_ptr(),
-                       (const float*)bx.data_ptr(), (float*)state.data_ptr(),
-                       (const int*)start_loc.data_ptr(), (const int*)slots.data_ptr(),
-                       (const int*)positions.data_ptr(), n);
+                       (const float*)bx.data_ptr(), (float*)state.data_ptr(), segA,
+                       segB, (const int*)start_loc.data_ptr(),
+                       (const int*)slots.data_ptr(),
+                       (const int*)positions.data_ptr(), n, nseg);
   });
   SEQ_CHECK_LAUNCH();
 }
+
+#define SEQ_SCAN_CASE(KQ)                                                     \
+  case KQ:                                                                    \
+    if (per_token) launch(linear_attn_scan_reg_kernel<act_t, true, KQ>);      \
+    else launch(linear_attn_scan_reg_kernel<act_t, false, KQ>);               \
+    break;
 
 void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                       torch::Tensor v, torch::Tensor decay,
@@ -186,6 +349,32 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   }
   const int n_seq = slots.numel();
   if (n_seq == 0 || T == 0) return;
+  if (D % 16 == 0 && D <= 128) {
+    const int ncb = (Dv + 15) / 16;
+    SEQ_DISPATCH_ACT(q, {
+      auto launch = [&](auto kern) {
+        hipLaunchKernelGGL(kern, dim3(n_seq * H * ncb), dim3(WAVE), 0, SEQ_STREAM(),
+                           (float*)o.data_ptr(), (const act_t*)q.data_ptr(),
+                           q.stride(0), (const act_t*)k.data_ptr(), k.stride(0),
+                           (const act_t*)v.data_ptr(), v.stride(0),
+                           per_token ? (const act_t*)decay.data_ptr() : nullptr,
+                           per_token ? decay.stride(0) : 0,
+                           per_token ? nullptr : (const float*)decay.data_ptr(),
+                           per_token ? (const float*)bonus->data_ptr() : nullptr,
+                           per_token ? (const float*)w_bias->data_ptr() : nullptr,
+                           (float*)state.data_ptr(), (const int*)start_loc.data_ptr(),
+                           (const int*)slots.data_ptr(),
+                           (const int*)positions.data_ptr(), H, Dv, ncb,
+                           silu_inputs ? 1 : 0);
+      };
+      switch (D / 16) {
+        SEQ_SCAN_CASE(1) SEQ_SCAN_CASE(2) SEQ_SCAN_CASE(3) SEQ_SCAN_CASE(4)
+        SEQ_SCAN_CASE(5) SEQ_SCAN_CASE(6) SEQ_SCAN_CASE(7) SEQ_SCAN_CASE(8)
+      }
+    });
+    SEQ_CHECK_LAUNCH();
+    return;
+  }
   const int threads = ((Dv + WAVE - 1) / WAVE) * WAVE;
   TORCH_CHECK(threads <= 1024, "value size too large");
   const size_t lds =
@@ -193,9 +382,18 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   TORCH_CHECK(lds <= 160 * 1024, "head state does not fit LDS");
   SEQ_DISPATCH_ACT(q, {
     auto launch = [&](auto kern) {
-      if (lds > 48 * 1024)
-        hipFuncSetAttribute((const void*)kern,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      // raise the dynamic-LDS cap once per kernel, outside any capture
+      static thread_local const void* raised[4] = {nullptr, nullptr, nullptr, nullptr};
+      if (lds > 48 * 1024) {
+        bool seen = false;
+        for (auto p : raised) seen |= p == (const void*)kern;
+        if (!seen) {
+          hipFuncSetAttribute((const void*)kern,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+          for (auto& p : raised)
+            if (p == nullptr) { p = (const void*)kern; break; }
+        }
+      }
       hipLaunchKernelGGL(kern, dim3(n_seq * H), dim3(threads), lds, SEQ_STREAM(),
                          (float*)o.data_ptr(), (const act_t*)q.data_ptr(),
                          q.stride(0), (const act_t*)k.data_ptr(), k.stride(0),

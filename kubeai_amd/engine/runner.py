@@ -41,7 +41,25 @@ class _DecodeGraph:
         )
         self.seq_lens = torch.ones(b_pad, dtype=torch.int32, device=dev)
         logits_idx = torch.arange(b_pad, dtype=torch.int64, device=dev)
+        # models with per-sequence state: every row is a one-token run; the
+        # rows' state slots are one more refreshed input (-1 on pad rows)
+        self.state_slots = None
+        seq = None
+        if runner.has_seq_state:
+            from kubeai_amd.ops.seq import SeqMeta
+
+            self.state_slots = torch.full((b_pad,), -1, dtype=torch.int32, device=dev)
+            seq = SeqMeta(
+                start_loc=torch.arange(b_pad + 1, dtype=torch.int32, device=dev),
+                slots=self.state_slots,
+                token_seq=torch.arange(b_pad, dtype=torch.int32, device=dev),
+                positions=self.positions,
+                block_tables=self.block_tables,
+                n_seq=b_pad,
+                max_len=1,
+            )
         self.fb = ForwardBatch(
+            seq=seq,
             input_ids=self.input_ids,
             positions=self.positions,
             slot_mapping=self.slots,
@@ -65,8 +83,14 @@ class _DecodeGraph:
             h = runner.model(self.fb)
             self.logits = runner.model.compute_logits(h[logits_idx])
 
-    def run(self, input_ids, positions, slots, tables, seq_lens) -> torch.Tensor:
+    def run(self, input_ids, positions, slots, tables, seq_lens,
+            state_slots=None) -> torch.Tensor:
         b = len(input_ids)
+        if self.state_slots is not None:
+            self.state_slots[:b].copy_(state_slots, non_blocking=True)
+            if b < self.b_pad:
+                self.state_slots[b:].fill_(-1)
+                self.positions[b:].fill_(0)
         self.input_ids[:b].copy_(input_ids, non_blocking=True)
         self.positions[:b].copy_(positions, non_blocking=True)
         self.slots[:b].copy_(slots, non_blocking=True)
@@ -487,6 +511,13 @@ class ModelRunner:
             torch.tensor(slots, dtype=torch.int64),
             torch.from_numpy(tables),
             torch.tensor(lens, dtype=torch.int32),
+            state_slots=(
+                torch.tensor(
+                    [ss.req.state_slot for ss in out.decode], dtype=torch.int32
+                )
+                if self.has_seq_state
+                else None
+            ),
         )
 
     @torch.inference_mode()
@@ -507,7 +538,6 @@ class ModelRunner:
         logits = None
         if (
             self.enable_graphs
-            and not self.has_seq_state
             and not out.prefill
             and out.decode
             and not (

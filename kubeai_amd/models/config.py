@@ -658,3 +658,43 @@ PRESETS: dict[str, ModelArchConfig] = {
         num_experts_per_tok=2,
     ),
 }
+
+
+def dulotar_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
+                   chunk: int = 1024, ff_mult: int = 4) -> ModelArchConfig:
+    """A Dulotar stack of the given size with random-init weights: the
+    pattern (wkv, mingru, parallel + feed-forward) repeated; sizes follow
+    common practice (head_dim-wide heads, 4:1 grouped keys, ff = 4 x width)."""
+    heads = max(1, width // head_dim)
+    kv = max(1, heads // 4)
+    lin_dim = min(head_dim, 128)
+    pattern = [
+        {"type": "wkv", "mlp": None,
+         "mixer": {"heads": max(1, width // 64), "dim": 64, "lowrank": max(16, width // 32)}},
+        {"type": "mingru", "mlp": None, "mixer": {"width": width}},
+        {"type": "parallel", "mlp": {"kind": "dense", "ff": ff_mult * width},
+         "mixer": {
+             "left": {"heads": heads, "kv_heads": kv, "dim": head_dim, "vdim": head_dim,
+                      "conv": 4, "mask": {"size": chunk},
+                      "rot": {"base": 10000.0, "dims": head_dim // 2},
+                      "scale": head_dim ** -0.5, "softcap": 50.0},
+             "left_scale": 1.0,
+             "right": {"heads": heads, "dim": lin_dim, "vdim": head_dim,
+                       "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(1, heads - 1))
+                                 for i in range(heads)]},
+             "right_scale": 1.0}},
+    ]
+    return dulotar_arch_config({
+        "architecture": "Dulotar", "vocab": vocab, "width": width,
+        "canon": {"taps": 4}, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+        "layers": [dict(pattern[i % 3]) for i in range(layers)],
+    })
+
+
+PRESETS.update({
+    "dulotar-tiny": dulotar_preset(128, 3, vocab=512, head_dim=32, chunk=64),
+    "dulotar-1k": dulotar_preset(1024, 12),
+    "dulotar-2k": dulotar_preset(2048, 12),
+    "dulotar-4k": dulotar_preset(4096, 6),
+})
+

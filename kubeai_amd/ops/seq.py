@@ -226,7 +226,7 @@ def mingru_scan(zxg, bz, bx, state, meta: SeqMeta):
         _require_ext()
         y = torch.empty((zxg.shape[0], n), dtype=zxg.dtype, device=zxg.device)
         _C.mingru_scan(y, zxg, bz, bx, state, meta.start_loc, meta.slots,
-                       meta.positions)
+                       meta.positions, meta.max_len)
         return y
     y = torch.empty((zxg.shape[0], n), dtype=zxg.dtype)
     for s0, ln, slot, p0 in meta.runs():

@@ -409,6 +409,39 @@ def test_greedy_generation_through_scheduler(tmp_path, device):
     assert eng.block_manager.num_free_blocks == eng.block_manager.num_blocks
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graph_replays_match_oracle(tmp_path, dtype):
+    """Pure-decode steps replay a captured graph; prompt portions of later
+    arrivals run eagerly between replays. Every generated token is checked."""
+    d, W = model_dir(tmp_path, MIXED, seed=17)
+    eng = LLMEngine(EngineConfig(
+        model=d, device="cuda", dtype=dtype, num_gpu_blocks=64, max_num_seqs=6,
+        max_model_len=512, max_num_batched_tokens=64, enable_graphs=True))
+    prompts = {"g%d" % i: tokens(n, MIXED["vocab"], 90 + i)
+               for i, n in enumerate([9, 33, 4, 70, 18, 2, 25])}
+    pending = list(prompts.items())
+    done, steps = {}, 0
+    while (pending or eng.has_work()) and steps < 500:
+        if pending and steps % 5 == 0:  # arrivals interleave with decode steps
+            rid, t = pending.pop(0)
+            eng.add_request(t, SamplingParams(max_tokens=24, ignore_eos=True),
+                            request_id=rid)
+        for o in eng.step():
+            if o.finished:
+                done[o.request_id] = list(o.output_token_ids)
+        steps += 1
+    assert eng.runner._graphs, "no decode graph was captured"
+    assert set(done) == set(prompts)
+    tol = 1e-3 if dtype == "float32" else 0.25
+    for rid, t in prompts.items():
+        gen = done[rid]
+        logits = oracle.forward(MIXED, W, t + gen)
+        for i, tok in enumerate(gen):
+            row = logits[len(t) - 1 + i]
+            assert row[tok] >= row.max() - tol * row.std(), (rid, i)
+
+
 def test_state_slots_survive_preemption_and_abort(tmp_path):
     d, W = model_dir(tmp_path, MIXED, seed=16)
     eng = LLMEngine(EngineConfig(

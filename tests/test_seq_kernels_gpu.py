@@ -11,9 +11,14 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
 
 
+RUNS = "short"
+
+
 def _meta(device, block_tables=None):
     # (length, slot, first position)
     runs = [(1, 2, 37), (1, 0, 5), (19, 3, 0), (7, 1, 30), (2, 5, 64), (5, -1, 0)]
+    if RUNS == "long":  # runs that span several scan segments / staging tiles
+        runs = [(1, 2, 37), (200, 3, 0), (130, 1, 77), (64, 4, 5), (65, 0, 0), (3, -1, 0)]
     pos = torch.cat([torch.arange(p, p + n) for n, _, p in runs]).int()
     return sops.SeqMeta.build([(n, s) for n, s, _ in runs], pos.to(device), device,
                               block_tables=block_tables), int(pos.numel())
@@ -107,8 +112,16 @@ def test_token_shift_mix(dtype):
     torch.testing.assert_close(gs[0].cpu(), cs[0], atol=1e-6, rtol=1e-6)
 
 
+@pytest.fixture(params=["short", "long"])
+def runs(request):
+    global RUNS
+    RUNS = request.param
+    yield request.param
+    RUNS = "short"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_mingru_scan(dtype):
+def test_mingru_scan(dtype, runs):
     torch.manual_seed(4)
     _, T = _meta("cpu")
     n = 300
@@ -118,12 +131,13 @@ def test_mingru_scan(dtype):
     fn = lambda meta, zxg, bz, bx, st: sops.mingru_scan(zxg, bz, bx, st, meta)
     c, g, cs, gs = _both(fn, dtype, [zxg, bz, bx], [st])
     torch.testing.assert_close(g.cpu().float(), c.float(), **_tol(dtype))
-    torch.testing.assert_close(gs[0].cpu(), cs[0], atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(gs[0].cpu(), cs[0], atol=1e-4, rtol=1e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,Dv", [(2, 48, 48), (3, 16, 80), (1, 64, 64)])
-def test_linear_attn_scan_per_token_decay(dtype, H, D, Dv):
+@pytest.mark.parametrize("H,D,Dv", [(2, 48, 48), (3, 16, 80), (1, 64, 64), (2, 128, 128),
+                                    (2, 40, 40)])
+def test_linear_attn_scan_per_token_decay(dtype, H, D, Dv, runs):
     if D != Dv:
         pytest.skip("bonus form pairs equal key/value sizes in the model; "
                     "unequal sizes are covered by the constant-decay form")
@@ -146,12 +160,13 @@ def test_linear_attn_scan_per_token_decay(dtype, H, D, Dv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,Dv", [(4, 64, 64), (3, 16, 80), (2, 40, 24)])
-def test_linear_attn_scan_constant_decay(dtype, H, D, Dv):
+@pytest.mark.parametrize("H,D,Dv", [(4, 64, 64), (3, 16, 80), (2, 40, 24), (2, 32, 24),
+                                    (1, 112, 130)])
+def test_linear_attn_scan_constant_decay(dtype, H, D, Dv, runs):
     torch.manual_seed(6)
     _, T = _meta("cpu")
-    q = torch.randn(T, H, D).to(dtype)
-    k = torch.randn(T, H, D).to(dtype)
+    q = (torch.randn(T, H, D) * 0.5).to(dtype)
+    k = (torch.randn(T, H, D) * 0.5).to(dtype)
     v = torch.randn(T, H, Dv).to(dtype)
     dec = torch.rand(H) * 0.5 + 0.5
     st = torch.randn(6, H, D, Dv)
