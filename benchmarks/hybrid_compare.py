@@ -12,6 +12,7 @@ measurement on stdout.
 from __future__ import annotations
 
 import json
+import sys
 import time
 
 import torch
@@ -20,6 +21,10 @@ from kubeai_amd.models.config import PRESETS, ModelArchConfig
 
 SIZES = {"1k": ("dulotar-1k", 1024, 12), "2k": ("dulotar-2k", 2048, 12),
          "4k": ("dulotar-4k", 4096, 6)}
+
+
+def _log(msg: str) -> None:
+    print(f"[compare t={time.monotonic():.1f}] {msg}", file=sys.stderr, flush=True)
 
 
 def _params(model) -> int:
@@ -114,6 +119,7 @@ def main(args) -> None:
         arch = PRESETS[name]
         max_len = 8192 + 256
         blocks = (max(b * (c + 128) for b, c in batches) + max_len) // 16 + 64
+        _log(f"dulotar {key}: building engine ({name})")
         eng = _engine(name, device, blocks, 64, max_len)
         n_params = _params(eng.runner.model)
         ref_name = f"llama-like-{key}"
@@ -127,11 +133,13 @@ def main(args) -> None:
                 eng = _engine(model_name, device, blocks, 64, max_len)
             params = _params(eng.runner.model)
             for n in prefill_lens:
+                _log(f"{fam} {key}: prefill {n}")
                 tps = _prefill(eng, device, arch.vocab_size, n)
                 print(json.dumps({"bench": "prefill", "family": fam, "size": key,
                                   "params_m": round(params / 1e6, 1), "tokens": n,
                                   "tokens_per_s": round(tps, 1)}), flush=True)
             for b, c in batches:
+                _log(f"{fam} {key}: decode batch {b} context {c}")
                 tps, ms = _decode(eng, device, arch.vocab_size, b, c)
                 print(json.dumps({"bench": "decode", "family": fam, "size": key,
                                   "params_m": round(params / 1e6, 1), "batch": b,

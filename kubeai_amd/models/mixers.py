@@ -90,7 +90,7 @@ class WKVMixer(nn.Module):
         self.width, self.heads, self.dim, self.eps = width, heads, dim, eps
         n = heads * dim
         self.mu = _f32(5, width)
-        # r, k, v, g share the output size: one batched GEMM over four mixes
+        # r, k, v, g share the output size: stacked [4, n, width]
         self.rkvg = nn.Parameter(torch.empty(4, n, width), requires_grad=False)
         nn.init.normal_(self.rkvg, std=width ** -0.5)
         self.w1 = Proj(width, lowrank)
@@ -110,7 +110,9 @@ class WKVMixer(nn.Module):
         T = h.shape[0]
         H, D = self.heads, self.dim
         mixes = sops.token_shift_mix(h, self.mu, state["prev"], fb.seq)
-        rkvg = torch.bmm(mixes[:4], self.rkvg.transpose(1, 2))  # [4, T, n]
+        # four plain GEMMs (the library path every other family uses; the
+        # strided-batched path is not exercised under the tuned-GEMM table)
+        rkvg = [F.linear(mixes[i], self.rkvg[i]) for i in range(4)]
         lr = torch.tanh(self.w1(mixes[4]).float()).to(h.dtype)
         wpre = self.w2(lr)
         o = sops.linear_attn_scan(
