@@ -195,27 +195,74 @@ __global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
     U[i] = kPerToken ? bonus[h * D + r * R + i] : 0.f;
   }
   const float dc = kPerToken ? 0.f : decay_const[h];
+  // staging: lane (st_tt, st_part) owns a quarter row of one token of the
+  // tile; the next tile's vectors are fetched into registers while the
+  // current tile is walked, so the lone wave never waits on memory
+  typedef typename Raw4<T>::type raw4;
+  const int st_tt = lane >> 2, st_part = lane & 3;
+  raw4 pq[kQ], pk[kQ], pw[kQ];
+  T pv[4];
+  float wb[kPerToken ? R : 1];
+  if (kPerToken) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) wb[i] = w_bias[h * D + st_part * R + i];
+  }
+  auto prefetch = [&](int tile0) {
+    const int t = tile0 + st_tt;
+    if (t < s1) {
+      const T* qp = q + (size_t)t * q_stride + h * D + st_part * R;
+      const T* kp = k + (size_t)t * k_stride + h * D + st_part * R;
+#pragma unroll
+      for (int b = 0; b < kQ; ++b) {
+        pq[b] = *(const raw4*)(qp + 4 * b);
+        pk[b] = *(const raw4*)(kp + 4 * b);
+      }
+      if (kPerToken) {
+        const T* wp = decay_pre + (size_t)t * d_stride + h * D + st_part * R;
+#pragma unroll
+        for (int b = 0; b < kQ; ++b) pw[b] = *(const raw4*)(wp + 4 * b);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int col = cb * 16 + st_part * 4 + e;
+        pv[e] = col < Dv ? v[(size_t)t * v_stride + h * Dv + col] : (T)0;
+      }
+    }
+  };
+  prefetch(s0);
   for (int t0 = s0; t0 < s1; t0 += kScanTile) {
     const int nt = min(kScanTile, s1 - t0);
     __syncthreads();
-    for (int i = lane; i < nt * D; i += WAVE) {
-      const int tt = i / D, d = i % D;
-      float qv = ldf(q + (size_t)(t0 + tt) * q_stride + h * D + d);
-      float kv = ldf(k + (size_t)(t0 + tt) * k_stride + h * D + d);
-      if (silu_inputs) { qv = silu_f(qv); kv = silu_f(kv); }
-      qs[i] = qv;
-      ks[i] = kv;
-      if (kPerToken)
-        ws[i] = expf(-expf(ldf(decay_pre + (size_t)(t0 + tt) * d_stride + h * D + d) +
-                           w_bias[h * D + d]));
-    }
-    for (int i = lane; i < nt * 16; i += WAVE) {
-      const int tt = i / 16, cc = cb * 16 + (i % 16);
-      float vv = cc < Dv ? ldf(v + (size_t)(t0 + tt) * v_stride + h * Dv + cc) : 0.f;
-      if (silu_inputs) vv = silu_f(vv);
-      vs[i] = vv;
+    if (st_tt < nt) {
+#pragma unroll
+      for (int b = 0; b < kQ; ++b) {
+        float a[4], bb[4];
+        cvt4(pq[b], a);
+        cvt4(pk[b], bb);
+        if (silu_inputs) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { a[e] = silu_f(a[e]); bb[e] = silu_f(bb[e]); }
+        }
+        const int at = st_tt * D + st_part * R + 4 * b;
+        *(float4*)(qs + at) = make_float4(a[0], a[1], a[2], a[3]);
+        *(float4*)(ks + at) = make_float4(bb[0], bb[1], bb[2], bb[3]);
+        if (kPerToken) {
+          float w[4];
+          cvt4(pw[b], w);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = expf(-expf(w[e] + wb[4 * b + e]));
+          *(float4*)(ws + at) = make_float4(w[0], w[1], w[2], w[3]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float vv = ldf(&pv[e]);
+        if (silu_inputs) vv = silu_f(vv);
+        vs[st_tt * 16 + st_part * 4 + e] = vv;
+      }
     }
     __syncthreads();
+    if (t0 + kScanTile < s1) prefetch(t0 + kScanTile);
     for (int tt = 0; tt < nt; ++tt) {
       const float vj = vs[tt * 16 + c];
       const float4* q4 = (const float4*)(qs + tt * D + r * R);
@@ -349,7 +396,12 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   }
   const int n_seq = slots.numel();
   if (n_seq == 0 || T == 0) return;
-  if (D % 16 == 0 && D <= 128) {
+  auto vec_ok = [&](const torch::Tensor& t) {
+    const size_t bytes = 4 * t.element_size();
+    return ((size_t)t.data_ptr()) % bytes == 0 && t.stride(0) % 4 == 0;
+  };
+  const bool aligned = vec_ok(q) && vec_ok(k) && (!per_token || vec_ok(decay));
+  if (D % 16 == 0 && D <= 128 && aligned) {
     const int ncb = (Dv + 15) / 16;
     SEQ_DISPATCH_ACT(q, {
       auto launch = [&](auto kern) {

@@ -30,6 +30,19 @@ DEV_INLINE float ldf(const bf16raw* p) { return bf16_to_f32(*p); }
 DEV_INLINE void stf(float* p, float v) { *p = v; }
 DEV_INLINE void stf(bf16raw* p, float v) { *p = f32_to_bf16(v); }
 
+// four consecutive activations as one vector load (pointer aligned to four
+// elements), kept raw until they are needed
+template <typename T> struct Raw4;
+template <> struct Raw4<float> { typedef float4 type; };
+template <> struct Raw4<bf16raw> { typedef ushort4 type; };
+DEV_INLINE void cvt4(const float4& v, float* o) {
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+DEV_INLINE void cvt4(const ushort4& v, float* o) {
+  o[0] = bf16_to_f32(v.x); o[1] = bf16_to_f32(v.y);
+  o[2] = bf16_to_f32(v.z); o[3] = bf16_to_f32(v.w);
+}
+
 DEV_INLINE float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 DEV_INLINE float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
