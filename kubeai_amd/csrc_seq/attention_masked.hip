@@ -132,6 +132,128 @@ __global__ __launch_bounds__(WAVE) void masked_paged_attention_kernel(
   }
 }
 
+typedef __attribute__((ext_vector_type(4))) short bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kMaxDSteps = 8;    // key size <= 128
+constexpr int kMaxDvTiles = 16;  // value size <= 256
+
+// Prompt portions on the matrix cores (bf16, key and value sizes multiples
+// of 16). grid (n_seq * tiles_per_run, H), one wave per 16 consecutive
+// queries of a run and one query head. Per 16-key tile:
+//   S^T = K Q^T   (v_mfma_f32_16x16x16_bf16, K rows straight from the cache)
+//   fp32 scale, cap, mask, running max / sum per query (a query is a lane
+//   column, so its statistics never leave the lane quad 16 apart)
+//   O^T += V^T P^T with P^T taken from S^T's accumulator layout as is.
+__global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
+    bf16raw* __restrict__ out, int64_t out_stride, const bf16raw* __restrict__ q,
+    int64_t q_stride, const bf16raw* __restrict__ k_cache,
+    const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
+    int max_blocks, const int* __restrict__ start_loc,
+    const int* __restrict__ positions, int tiles_per_run, float scale,
+    float softcap, int chunk, int window, float out_scale, int H, int G, int D,
+    int Dv, int bs) {
+  const int s = blockIdx.x / tiles_per_run, tile = blockIdx.x % tiles_per_run;
+  const int h = blockIdx.y, g = h / (H / G);
+  const int s0 = start_loc[s], s1 = start_loc[s + 1];
+  const int q0 = s0 + tile * 16;
+  if (q0 >= s1) return;
+  const int nq = min(16, s1 - q0);
+  const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
+  const bool q_ok = col < nq;
+  const int tq = q0 + min(col, nq - 1);
+  const int pos_q = q_ok ? positions[tq] : -1;
+  const int pos_min = positions[q0], pos_max = pos_min + nq - 1;
+  auto lower = [&](int p) {
+    int lo = 0;
+    if (chunk > 0) lo = (p / chunk) * chunk;
+    if (window > 0) lo = max(lo, p - window + 1);
+    return lo;
+  };
+  const int lo_q = q_ok ? lower(pos_q) : 0;
+  const int lo_tile = lower(pos_min);
+  const int* bt = block_tables + (size_t)s * max_blocks;
+  const int nks = D / 16, ndt = Dv / 16;
+  bf16x4 qf[kMaxDSteps];
+#pragma unroll
+  for (int ks = 0; ks < kMaxDSteps; ++ks)
+    if (ks < nks)
+      qf[ks] = *(const bf16x4*)(q + (size_t)tq * q_stride + h * D + ks * 16 + grp * 4);
+  f32x4 oacc[kMaxDvTiles];
+#pragma unroll
+  for (int dt = 0; dt < kMaxDvTiles; ++dt) oacc[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  for (int j0 = lo_tile; j0 <= pos_max; j0 += 16) {
+    // K operand: row = key j0 + col, 4 consecutive dims per step
+    const int jk = min(j0 + col, pos_max);
+    const bf16raw* kp = k_cache + (((int64_t)bt[jk / bs] * G + g) * bs + jk % bs) * D + grp * 4;
+    f32x4 sacc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < kMaxDSteps; ++ks)
+      if (ks < nks)
+        sacc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+            *(const bf16x4*)(kp + ks * 16), qf[ks], sacc, 0, 0, 0);
+    // this lane: query `col`, keys j0 + grp * 4 + i
+    float sc[4];
+    bool vis[4];
+    int64_t vrow[4];
+    float mt = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = j0 + grp * 4 + i;
+      float x = sacc[i] * scale;
+      if (softcap > 0.f) x = softcap * tanhf(x / softcap);
+      vis[i] = j <= pos_q && j >= lo_q;
+      sc[i] = vis[i] ? x : -INFINITY;
+      mt = fmaxf(mt, sc[i]);
+      const int jv = min(j, pos_max);
+      vrow[i] = (((int64_t)bt[jv / bs] * G + g) * bs + jv % bs) * Dv;
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
+    const float m_new = fmaxf(m, mt);
+    const float corr = m_new == -INFINITY ? 1.f : expf(m - m_new);
+    bf16x4 pb;
+    float ps = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = vis[i] ? expf(sc[i] - m_new) : 0.f;
+      ps += p;
+      pb[i] = (short)f32_to_bf16(p);
+    }
+    l = l * corr + ps;
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < kMaxDvTiles; ++dt) {
+      if (dt < ndt) {
+        bf16x4 vf;  // V^T operand: row = value dim dt*16 + col, keys grp*4 + i
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vf[i] = (short)v_cache[vrow[i] + dt * 16 + col];
+        f32x4 a = oacc[dt];
+        a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
+        oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pb, a, 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (q_ok) {
+    const float inv = out_scale / l;
+    bf16raw* op = out + (size_t)tq * out_stride + h * Dv + grp * 4;
+#pragma unroll
+    for (int dt = 0; dt < kMaxDvTiles; ++dt) {
+      if (dt < ndt) {
+        ushort4 o4;
+        o4.x = f32_to_bf16(oacc[dt][0] * inv);
+        o4.y = f32_to_bf16(oacc[dt][1] * inv);
+        o4.z = f32_to_bf16(oacc[dt][2] * inv);
+        o4.w = f32_to_bf16(oacc[dt][3] * inv);
+        *(ushort4*)(op + dt * 16) = o4;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 static bool dense_heads3(const torch::Tensor& t) {
@@ -177,10 +299,11 @@ void rope_pairs_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
 
 void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor k_cache, torch::Tensor v_cache,
-                            torch::Tensor block_tables, torch::Tensor token_seq,
-                            torch::Tensor positions, double scale,
-                            double softcap, int64_t chunk, int64_t window,
-                            double out_scale) {
+                            torch::Tensor block_tables, torch::Tensor start_loc,
+                            torch::Tensor token_seq, torch::Tensor positions,
+                            int64_t max_len, double scale, double softcap,
+                            int64_t chunk, int64_t window, double out_scale) {
+  check_i32(start_loc, "start_loc");
   check_i32(block_tables, "block_tables");
   check_i32(token_seq, "token_seq");
   check_i32(positions, "positions");
@@ -199,6 +322,29 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
               v_cache.scalar_type() == q.scalar_type() &&
               out.scalar_type() == q.scalar_type());
   if (T == 0) return;
+  const int n_seq = start_loc.numel() - 1;
+  TORCH_CHECK(block_tables.size(0) >= n_seq);
+  auto al8 = [](const torch::Tensor& t) {
+    return ((size_t)t.data_ptr()) % 8 == 0 && t.stride(0) % 4 == 0;
+  };
+  if (q.scalar_type() == torch::kBFloat16 && max_len > 1 && D % 16 == 0 &&
+      Dv % 16 == 0 && D <= 16 * kMaxDSteps && Dv <= 16 * kMaxDvTiles && al8(q) &&
+      al8(out)) {
+    // prompt portions: matrix-core kernel over 16-query tiles of every run
+    const int tiles = (int)((max_len + 15) / 16);
+    hipLaunchKernelGGL(masked_prefill_mfma_kernel, dim3(n_seq * tiles, H),
+                       dim3(WAVE), 0, SEQ_STREAM(), (bf16raw*)out.data_ptr(),
+                       out.stride(0), (const bf16raw*)q.data_ptr(), q.stride(0),
+                       (const bf16raw*)k_cache.data_ptr(),
+                       (const bf16raw*)v_cache.data_ptr(),
+                       (const int*)block_tables.data_ptr(),
+                       (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
+                       (const int*)positions.data_ptr(), tiles, (float)scale,
+                       (float)softcap, (int)chunk, (int)window, (float)out_scale, H,
+                       G, D, Dv, bs);
+    SEQ_CHECK_LAUNCH();
+    return;
+  }
   const size_t lds = (size_t)(D + WAVE) * 4 + WAVE * 8;
   SEQ_DISPATCH_ACT(q, {
     hipLaunchKernelGGL((masked_paged_attention_kernel<act_t>), dim3(T, H),

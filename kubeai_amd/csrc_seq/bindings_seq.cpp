@@ -31,10 +31,10 @@ void rope_pairs_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                           torch::Tensor slot_mapping);
 void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor k_cache, torch::Tensor v_cache,
-                            torch::Tensor block_tables, torch::Tensor token_seq,
-                            torch::Tensor positions, double scale,
-                            double softcap, int64_t chunk, int64_t window,
-                            double out_scale);
+                            torch::Tensor block_tables, torch::Tensor start_loc,
+                            torch::Tensor token_seq, torch::Tensor positions,
+                            int64_t max_len, double scale, double softcap,
+                            int64_t chunk, int64_t window, double out_scale);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_layernorm", &add_layernorm, "fp32 residual add + LayerNorm");

@@ -347,8 +347,9 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
     if q.is_cuda:
         _require_ext()
         _C.masked_paged_attention(out, q, k_cache, v_cache, meta.block_tables,
-                                  meta.token_seq, meta.positions, scale,
-                                  softcap, chunk, window, out_scale)
+                                  meta.start_loc, meta.token_seq, meta.positions,
+                                  meta.max_len, scale, softcap, chunk, window,
+                                  out_scale)
         return out
     T, H, D = q.shape
     G, bs = k_cache.shape[1], k_cache.shape[2]

@@ -180,13 +180,25 @@ def test_long_decoding(tmp_path, device):
     check(replay(engine(d, device), "a", toks, [9, 1]), want)
 
 
+# sizes in multiples of 16: bf16 prompt portions take the matrix-core
+# attention kernel and the register-state scans
+MFMA_SIZED = config(
+    [wkv(heads=2, dim=16), gru(n=48, mlp=FF),
+     par(l=left(heads=4, kv=2, dim=32, vdim=16, conv=3, size=24, rot=16, scale=0.18),
+         r=right(heads=2, dim=16, vdim=32, decay=(0.9, 0.99)), mlp=FF)],
+    width=64, vocab=80)
+
+
 @pytest.mark.parametrize("device", [pytest.param("cuda", marks=pytest.mark.gpu)])
-def test_bfloat16_serving_precision(tmp_path, device):
-    d, W = model_dir(tmp_path, MIXED, seed=8)
-    toks = tokens(60, MIXED["vocab"], 6)
-    want = oracle.forward(MIXED, W, toks)
-    got = replay(engine(d, device, dtype="bfloat16"), "a", toks, [17, 2, 1])
+@pytest.mark.parametrize("cfg", [MIXED, MFMA_SIZED], ids=["odd_sizes", "sixteens"])
+def test_bfloat16_serving_precision(tmp_path, device, cfg):
+    d, W = model_dir(tmp_path, cfg, seed=8)
+    toks = tokens(120, cfg["vocab"], 6)
+    want = oracle.forward(cfg, W, toks)
+    got = replay(engine(d, device, dtype="bfloat16"), "a", toks, [50, 17, 2, 1])
     check(got, want, dtype="bfloat16")
+    got = replay(engine(d, device, dtype="float32"), "b", toks, [50, 17, 2, 1])
+    check(got, want)
 
 
 # ---------------------------------------------------------------------------

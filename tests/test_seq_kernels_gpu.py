@@ -181,11 +181,15 @@ def test_linear_attn_scan_constant_decay(dtype, H, D, Dv, runs):
 @pytest.mark.parametrize("H,G,D,Dv,rot,chunk,window,cap",
                          [(8, 4, 48, 96, 48, 16, 0, 50.0), (4, 1, 32, 32, 16, 0, 0, 0.0),
                           (6, 2, 24, 130, 8, 40, 9, 5.0), (2, 2, 64, 64, 64, 0, 11, 0.0)])
-def test_rope_cache_and_masked_attention(dtype, H, G, D, Dv, rot, chunk, window, cap):
+@pytest.mark.parametrize("long_runs", [False, True])
+def test_rope_cache_and_masked_attention(dtype, H, G, D, Dv, rot, chunk, window, cap,
+                                         long_runs):
     torch.manual_seed(7)
-    bs, nblk = 16, 40
+    bs, nblk = 16, 60
     runs = [(1, 2, 37), (1, 0, 5), (19, 3, 0), (7, 1, 30), (2, 5, 64), (5, -1, 0)]
-    tables = torch.zeros(len(runs), 6, dtype=torch.int32)
+    if long_runs:  # several 16-query tiles, chunk edges inside a tile
+        runs = [(1, 2, 37), (150, 3, 0), (77, 1, 130), (33, 4, 15), (5, -1, 0)]
+    tables = torch.zeros(len(runs), 14, dtype=torch.int32)
     free = list(torch.randperm(nblk - 1).add(1).tolist())
     for i, (n, s, p) in enumerate(runs):
         if s >= 0:
