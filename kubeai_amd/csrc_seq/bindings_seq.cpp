@@ -24,7 +24,7 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                       c10::optional<torch::Tensor> bonus,
                       c10::optional<torch::Tensor> w_bias, torch::Tensor state,
                       torch::Tensor start_loc, torch::Tensor slots,
-                      torch::Tensor positions, bool silu_inputs);
+                      torch::Tensor positions, bool silu_inputs, int64_t max_len);
 void rope_pairs_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                           torch::Tensor positions, torch::Tensor inv_freq,
                           torch::Tensor k_cache, torch::Tensor v_cache,

@@ -172,13 +172,23 @@ __global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
     const float* __restrict__ w_bias, float* __restrict__ state,
     const int* __restrict__ start_loc, const int* __restrict__ slots,
     const int* __restrict__ positions, int H, int Dv, int ncb,
-    int silu_inputs) {
+    int silu_inputs, int nseg, int seg_len, int compose,
+    float* __restrict__ segB, float* __restrict__ segW) {
   constexpr int R = 4 * kQ, D = 4 * R;
   const int cb = blockIdx.x % ncb;
   const int h = (blockIdx.x / ncb) % H;
-  const int s = blockIdx.x / (ncb * H);
-  const int s0 = start_loc[s], s1 = start_loc[s + 1], slot = slots[s];
-  if (s1 <= s0) return;
+  const int seg = (blockIdx.x / (ncb * H)) % nseg;
+  const int s = blockIdx.x / (ncb * H * nseg);
+  const int r0 = start_loc[s], s1_run = start_loc[s + 1], slot = slots[s];
+  // Long runs are cut into segments of seg_len tokens that run in parallel.
+  // The state update is affine in the state, S -> diag(W) S + B, so pass 1
+  // (compose) walks every segment but the last from zero and stores its
+  // (W, B); pass 2 folds the earlier segments into the incoming state and
+  // walks its own segment again, now writing the outputs.
+  const int s0 = r0 + seg * seg_len;
+  const int s1 = min(s0 + seg_len, s1_run);
+  if (s0 >= s1_run) return;
+  if (compose && s1 == s1_run) return;
   __shared__ __attribute__((aligned(16))) float qs[kScanTile * D];
   __shared__ __attribute__((aligned(16))) float ks[kScanTile * D];
   __shared__ __attribute__((aligned(16))) float ws[kPerToken ? kScanTile * D : 4];
@@ -186,15 +196,30 @@ __global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
   const int lane = threadIdx.x, r = lane >> 4, c = lane & 15;
   const int j = cb * 16 + c;
   const bool valid = j < Dv;
-  const bool carry = slot >= 0 && positions[s0] > 0;
+  const bool carry = !compose && slot >= 0 && positions[r0] > 0;
   float* sp = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * D * Dv;
-  float S[R], U[R];
+  float S[R], U[R], Wp[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     S[i] = (carry && valid) ? sp[(size_t)(r * R + i) * Dv + j] : 0.f;
     U[i] = kPerToken ? bonus[h * D + r * R + i] : 0.f;
+    Wp[i] = 1.f;
   }
   const float dc = kPerToken ? 0.f : decay_const[h];
+  if (!compose && seg > 0) {
+    float wfull = 1.f;  // constant decay over one full segment
+    if (!kPerToken)
+      for (int n = 0; n < seg_len; ++n) wfull *= dc;
+    for (int gg = 0; gg < seg; ++gg) {
+      const size_t base = ((size_t)(s * nseg + gg) * H + h) * D;
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        const float w = kPerToken ? segW[base + r * R + i] : wfull;
+        const float b = valid ? segB[(base + r * R + i) * Dv + j] : 0.f;
+        S[i] = w * S[i] + b;
+      }
+    }
+  }
   // staging: lane (st_tt, st_part) owns a quarter row of one token of the
   // tile; the next tile's vectors are fetched into registers while the
   // current tile is walked, so the lone wave never waits on memory
@@ -286,6 +311,7 @@ __global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
           if (kPerToken) {
             acc += qa[e] * (S[i] + U[i] * kv);
             S[i] = wa[e] * S[i] + kv;
+            if (compose) Wp[i] *= wa[e];
           } else {
             S[i] = dc * S[i] + kv;
             acc += qa[e] * S[i];
@@ -294,10 +320,17 @@ __global__ __launch_bounds__(WAVE) void linear_attn_scan_reg_kernel(
       }
       acc += __shfl_xor(acc, 16, WAVE);
       acc += __shfl_xor(acc, 32, WAVE);
-      if (r == 0 && valid) o[((size_t)(t0 + tt) * H + h) * Dv + j] = acc;
+      if (!compose && r == 0 && valid) o[((size_t)(t0 + tt) * H + h) * Dv + j] = acc;
     }
   }
-  if (slot >= 0 && valid) {
+  if (compose) {
+    const size_t base = ((size_t)(s * nseg + seg) * H + h) * D;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (valid) segB[(base + r * R + i) * Dv + j] = S[i];
+      if (kPerToken && cb == 0 && c == 0) segW[base + r * R + i] = Wp[i];
+    }
+  } else if (slot >= 0 && valid && s1 == s1_run) {
 #pragma unroll
     for (int i = 0; i < R; ++i) sp[(size_t)(r * R + i) * Dv + j] = S[i];
   }
@@ -362,7 +395,7 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                       c10::optional<torch::Tensor> bonus,
                       c10::optional<torch::Tensor> w_bias, torch::Tensor state,
                       torch::Tensor start_loc, torch::Tensor slots,
-                      torch::Tensor positions, bool silu_inputs) {
+                      torch::Tensor positions, bool silu_inputs, int64_t max_len) {
   check_f32(o, "o");
   check_f32(state, "state");
   check_i32(start_loc, "start_loc");
@@ -403,9 +436,24 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   const bool aligned = vec_ok(q) && vec_ok(k) && (!per_token || vec_ok(decay));
   if (D % 16 == 0 && D <= 128 && aligned) {
     const int ncb = (Dv + 15) / 16;
+    // segment-parallel walk of long runs (see the kernel); the workspace
+    // holds every segment's composed (W, B)
+    int seg_len = 128, nseg = 1;
+    if (max_len > 2 * seg_len) {
+      nseg = (int)((max_len + seg_len - 1) / seg_len);
+      while ((size_t)n_seq * nseg * H * D * Dv * 4 > ((size_t)2 << 30)) {
+        seg_len *= 2;
+        nseg = (int)((max_len + seg_len - 1) / seg_len);
+      }
+    }
+    torch::Tensor wsB, wsW;
+    if (nseg > 1) {
+      wsB = torch::empty({(int64_t)n_seq * nseg * H * D * Dv}, state.options());
+      wsW = torch::empty({(int64_t)n_seq * nseg * H * D}, state.options());
+    }
     SEQ_DISPATCH_ACT(q, {
-      auto launch = [&](auto kern) {
-        hipLaunchKernelGGL(kern, dim3(n_seq * H * ncb), dim3(WAVE), 0, SEQ_STREAM(),
+      auto launch1 = [&](auto kern, int compose) {
+        hipLaunchKernelGGL(kern, dim3(n_seq * nseg * H * ncb), dim3(WAVE), 0, SEQ_STREAM(),
                            (float*)o.data_ptr(), (const act_t*)q.data_ptr(),
                            q.stride(0), (const act_t*)k.data_ptr(), k.stride(0),
                            (const act_t*)v.data_ptr(), v.stride(0),
@@ -417,7 +465,13 @@ void linear_attn_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                            (float*)state.data_ptr(), (const int*)start_loc.data_ptr(),
                            (const int*)slots.data_ptr(),
                            (const int*)positions.data_ptr(), H, Dv, ncb,
-                           silu_inputs ? 1 : 0);
+                           silu_inputs ? 1 : 0, nseg, seg_len, compose,
+                           nseg > 1 ? (float*)wsB.data_ptr() : nullptr,
+                           nseg > 1 ? (float*)wsW.data_ptr() : nullptr);
+      };
+      auto launch = [&](auto kern) {
+        if (nseg > 1) launch1(kern, 1);
+        launch1(kern, 0);
       };
       switch (D / 16) {
         SEQ_SCAN_CASE(1) SEQ_SCAN_CASE(2) SEQ_SCAN_CASE(3) SEQ_SCAN_CASE(4)

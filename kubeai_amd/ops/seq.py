@@ -265,7 +265,7 @@ def linear_attn_scan(q, k, v, decay, bonus, state, meta: SeqMeta, *,
         o = torch.empty((T, H, Dv), dtype=torch.float32, device=q.device)
         _C.linear_attn_scan(o, q, k, v, decay, bonus, w_bias, state,
                             meta.start_loc, meta.slots, meta.positions,
-                            silu_inputs)
+                            silu_inputs, meta.max_len)
         return o
     o = torch.empty((T, H, Dv), dtype=torch.float32)
     act = (lambda a: a * torch.sigmoid(a)) if silu_inputs else (lambda a: a)

@@ -18,7 +18,7 @@ def _meta(device, block_tables=None):
     # (length, slot, first position)
     runs = [(1, 2, 37), (1, 0, 5), (19, 3, 0), (7, 1, 30), (2, 5, 64), (5, -1, 0)]
     if RUNS == "long":  # runs that span several scan segments / staging tiles
-        runs = [(1, 2, 37), (200, 3, 0), (130, 1, 77), (64, 4, 5), (65, 0, 0), (3, -1, 0)]
+        runs = [(1, 2, 37), (700, 3, 0), (130, 1, 77), (64, 4, 5), (385, 0, 9), (3, -1, 0)]
     pos = torch.cat([torch.arange(p, p + n) for n, _, p in runs]).int()
     return sops.SeqMeta.build([(n, s) for n, s, _ in runs], pos.to(device), device,
                               block_tables=block_tables), int(pos.numel())
@@ -144,7 +144,7 @@ def test_linear_attn_scan_per_token_decay(dtype, H, D, Dv, runs):
     torch.manual_seed(5)
     _, T = _meta("cpu")
     wide = torch.randn(T, 3 * H * D + 8).to(dtype)
-    dec = (torch.randn(T, H, D) - 1).to(dtype)
+    dec = (torch.randn(T, H, D) - 2).to(dtype)
     u, w0 = torch.randn(H, D) * 0.5, torch.randn(H * D) * 0.5
     st = torch.randn(6, H, D, Dv)
 
