@@ -111,7 +111,7 @@ def main(args) -> None:
     device = "cuda" if torch.cuda.is_available() else "cpu"
     sizes = [s for s in (args.compare_sizes or "1k,2k,4k").split(",") if s]
     prefill_lens = [2048, 8192] if device == "cuda" else [64]
-    batches = [(64, 1024), (8, 4096)] if device == "cuda" else [(2, 32)]
+    batches = [(64, 1536), (8, 3584)] if device == "cuda" else [(2, 32)]
     for key in sizes:
         name, width, layers = SIZES[key]
         if device == "cpu":

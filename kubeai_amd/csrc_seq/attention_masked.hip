@@ -59,38 +59,58 @@ __global__ void rope_pairs_cache_kernel(
 
 constexpr int kMaxDvPerLane = 8;  // value size <= 512
 
-// grid (T, H), one wave per (token, query head). Keys are walked in tiles
-// of 64: each lane scores one key (fp32 dot, cap, mask), the wave keeps a
-// running max / sum, then lanes switch to value channels and accumulate
-// p . V for the tile. Serves single decode tokens and prompt portions alike
-// (every token reads its keys, including this step's, from the cache).
-template <typename T>
-__global__ __launch_bounds__(WAVE) void masked_paged_attention_kernel(
+constexpr int kDecWaves = 4;
+
+// grid (T, H), kDecWaves waves per (token, query head). Keys are walked in
+// tiles of 64, dealt round-robin to the waves (a decode token alone cannot
+// hide memory latency, so its keys are split): each lane scores one key
+// (fp32 dot, cap, mask), the wave keeps a running max / sum, then its lanes
+// turn to the values and accumulate p . V for the tile. The waves' partial
+// results are joined through LDS at the end. Serves single decode tokens
+// (and, in fp32 or at odd sizes, prompt portions): every token reads its
+// keys, this step's included, from the cache.
+//
+// kVec: key and value rows are read with 16-byte loads. For the values a
+// wave splits into 64 / (Dv / N) key groups, each lane owning N value
+// channels of its group's keys.
+template <typename T, bool kVec>
+__global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kernel(
     T* __restrict__ out, int64_t out_stride, const T* __restrict__ q,
     int64_t q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
     int window, float out_scale, int H, int G, int D, int Dv, int bs) {
+  constexpr int N = Vec16<T>::N;
+  const int lpr = kVec ? Dv / N : 1;          // lanes per value row
+  const int ngrp = kVec ? WAVE / lpr : 1;     // key groups of a wave
   extern __shared__ float sm[];
-  int64_t* vbase = (int64_t*)sm;          // [64] value row offsets
-  float* ps = sm + 2 * WAVE;              // [64] tile probabilities
-  float* qs = ps + WAVE;                  // [D]
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  int64_t* vbase = (int64_t*)sm + wave * WAVE;       // [waves][64] value row offsets
+  float* ps = sm + 2 * WAVE * kDecWaves + wave * WAVE;  // [waves][64] probabilities
+  float* stat = sm + 3 * WAVE * kDecWaves;           // [waves][2] max, sum
+  float* qs = stat + 2 * kDecWaves;                  // [D]
+  float* red_all = qs + ((D + 3) & ~3);              // [waves][groups][Dv]
+  float* red = red_all + (size_t)wave * ngrp * Dv;
+  const int t = blockIdx.x, h = blockIdx.y;
   const int g = h / (H / G);
   const int pos = positions[t];
   const int* bt = block_tables + (size_t)token_seq[t] * max_blocks;
   int lo = 0;
   if (chunk > 0) lo = (pos / chunk) * chunk;
   if (window > 0) lo = max(lo, pos - window + 1);
-  for (int i = lane; i < D; i += WAVE)
+  for (int i = threadIdx.x; i < D; i += blockDim.x)
     qs[i] = ldf(q + (size_t)t * q_stride + h * D + i);
   __syncthreads();
+  const int kg = lane / lpr, lv = lane % lpr;
+  const bool v_on = kVec && kg < ngrp;
   float m = -INFINITY, l = 0.f;
   float acc[kMaxDvPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxDvPerLane; ++i) acc[i] = 0.f;
-  for (int j0 = lo; j0 <= pos; j0 += WAVE) {
+  // the wave's own LDS rows are touched by this wave only, so the tile loop
+  // needs no block barrier (a wave's LDS accesses complete in order)
+  for (int j0 = lo + wave * WAVE; j0 <= pos; j0 += kDecWaves * WAVE) {
     const int j = j0 + lane;
     float sc = -INFINITY;
     int64_t vb = 0;
@@ -99,36 +119,91 @@ __global__ __launch_bounds__(WAVE) void masked_paged_attention_kernel(
       const int64_t rowi = (blk * G + g) * bs + (j % bs);
       const T* kp = k_cache + rowi * D;
       float dot = 0.f;
-      for (int i = 0; i < D; ++i) dot += qs[i] * ldf(kp + i);
+      if (kVec) {
+        for (int i = 0; i < D; i += N) {
+          float x[N];
+          Vec16<T>::load(kp + i, x);
+#pragma unroll
+          for (int e = 0; e < N; ++e) dot += qs[i + e] * x[e];
+        }
+      } else {
+        for (int i = 0; i < D; ++i) dot += qs[i] * ldf(kp + i);
+      }
       sc = dot * scale;
       if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
       vb = rowi * Dv;
     }
-    const float m_new = fmaxf(m, wave_max(sc));
+    const float m_new = fmaxf(m, wave_max(sc));  // finite: lane 0's key is visible
     const float p = j <= pos ? expf(sc - m_new) : 0.f;
-    const float corr = expf(m - m_new);  // m = -inf on the first tile -> 0
+    const float corr = expf(m - m_new);  // m = -inf on the wave's first tile -> 0
     l = l * corr + wave_sum(p);
     m = m_new;
-    __syncthreads();  // previous tile's readers are done
     ps[lane] = p;
     vbase[lane] = vb;
-    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's LDS writes landed
+    __builtin_amdgcn_wave_barrier();
     const int nk = min(WAVE, pos - j0 + 1);
+    if (kVec) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) acc[e] *= corr;
+      if (v_on) {
+        for (int jj = kg; jj < nk; jj += ngrp) {
+          float x[N];
+          Vec16<T>::load(v_cache + vbase[jj] + lv * N, x);
+          const float pj = ps[jj];
+#pragma unroll
+          for (int e = 0; e < N; ++e) acc[e] += pj * x[e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < kMaxDvPerLane; ++c) {
+        const int d = c * WAVE + lane;
+        if (d < Dv) {
+          float a = acc[c] * corr;
+          for (int jj = 0; jj < nk; ++jj) a += ps[jj] * ldf(v_cache + vbase[jj] + d);
+          acc[c] = a;
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // all lanes read ps/vbase before the next tile
+  }
+  // join: every wave publishes (max, sum) and its unnormalised partial output
+  if (lane == 0) {
+    stat[2 * wave] = m;
+    stat[2 * wave + 1] = l;
+  }
+  if (kVec) {
+    if (v_on) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) red[kg * Dv + lv * N + e] = acc[e];
+    }
+  } else {
 #pragma unroll
     for (int c = 0; c < kMaxDvPerLane; ++c) {
       const int d = c * WAVE + lane;
-      if (d < Dv) {
-        float a = acc[c] * corr;
-        for (int jj = 0; jj < nk; ++jj) a += ps[jj] * ldf(v_cache + vbase[jj] + d);
-        acc[c] = a;
-      }
+      if (d < Dv) red[d] = acc[c];
     }
   }
-  const float inv = out_scale / l;
-#pragma unroll
-  for (int c = 0; c < kMaxDvPerLane; ++c) {
-    const int d = c * WAVE + lane;
-    if (d < Dv) stf(out + (size_t)t * out_stride + h * Dv + d, acc[c] * inv);
+  __syncthreads();
+  float mx = -INFINITY;
+  for (int w = 0; w < kDecWaves; ++w) mx = fmaxf(mx, stat[2 * w]);
+  float wsc[kDecWaves], lsum = 0.f;
+  for (int w = 0; w < kDecWaves; ++w) {
+    const float mw = stat[2 * w];
+    wsc[w] = mw == -INFINITY ? 0.f : expf(mw - mx);  // a wave may have had no tile
+    lsum += stat[2 * w + 1] * wsc[w];
+  }
+  const float inv = out_scale / lsum;
+  for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
+    float a = 0.f;
+    for (int w = 0; w < kDecWaves; ++w) {
+      const float* rw = red_all + (size_t)w * ngrp * Dv;
+      float part = 0.f;
+      for (int gi = 0; gi < ngrp; ++gi) part += rw[gi * Dv + d];
+      a += part * wsc[w];
+    }
+    stf(out + (size_t)t * out_stride + h * Dv + d, a * inv);
   }
 }
 
@@ -345,18 +420,30 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
     SEQ_CHECK_LAUNCH();
     return;
   }
-  const size_t lds = (size_t)(D + WAVE) * 4 + WAVE * 8;
   SEQ_DISPATCH_ACT(q, {
-    hipLaunchKernelGGL((masked_paged_attention_kernel<act_t>), dim3(T, H),
-                       dim3(WAVE), lds, SEQ_STREAM(), (act_t*)out.data_ptr(),
-                       out.stride(0), (const act_t*)q.data_ptr(), q.stride(0),
-                       (const act_t*)k_cache.data_ptr(),
-                       (const act_t*)v_cache.data_ptr(),
-                       (const int*)block_tables.data_ptr(),
-                       (int)block_tables.size(1), (const int*)token_seq.data_ptr(),
-                       (const int*)positions.data_ptr(), (float)scale,
-                       (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                       H, G, D, Dv, bs);
+    constexpr int N = Vec16<act_t>::N;
+    // 16-byte row loads need whole vectors per key / value row and at most
+    // one wave of lanes per value row
+    const bool vec = D % N == 0 && Dv % N == 0 && Dv / N <= WAVE && Dv >= N &&
+                     N <= kMaxDvPerLane;
+    const int ngrp = vec ? WAVE / (Dv / N) : 1;
+    const size_t lds = (size_t)(3 * WAVE * kDecWaves + 2 * kDecWaves +
+                                ((D + 3) & ~3) + kDecWaves * ngrp * Dv) * 4;
+    TORCH_CHECK(lds <= 64 * 1024, "attention scratch exceeds LDS");
+    auto launch = [&](auto kern) {
+      hipLaunchKernelGGL(kern, dim3(T, H), dim3(kDecWaves * WAVE), lds, SEQ_STREAM(),
+                         (act_t*)out.data_ptr(), out.stride(0),
+                         (const act_t*)q.data_ptr(), q.stride(0),
+                         (const act_t*)k_cache.data_ptr(),
+                         (const act_t*)v_cache.data_ptr(),
+                         (const int*)block_tables.data_ptr(),
+                         (int)block_tables.size(1), (const int*)token_seq.data_ptr(),
+                         (const int*)positions.data_ptr(), (float)scale,
+                         (float)softcap, (int)chunk, (int)window, (float)out_scale,
+                         H, G, D, Dv, bs);
+    };
+    if (vec) launch(masked_paged_attention_kernel<act_t, true>);
+    else launch(masked_paged_attention_kernel<act_t, false>);
   });
   SEQ_CHECK_LAUNCH();
 }

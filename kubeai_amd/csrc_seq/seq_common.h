@@ -43,6 +43,28 @@ DEV_INLINE void cvt4(const ushort4& v, float* o) {
   o[2] = bf16_to_f32(v.z); o[3] = bf16_to_f32(v.w);
 }
 
+// one 16-byte load: 8 bf16 or 4 fp32 activations (pointer 16-byte aligned)
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+  static constexpr int N = 4;
+  static DEV_INLINE void load(const float* p, float* o) {
+    const float4 v = *(const float4*)p;
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+  }
+};
+template <> struct Vec16<bf16raw> {
+  static constexpr int N = 8;
+  static DEV_INLINE void load(const bf16raw* p, float* o) {
+    const uint4 v = *(const uint4*)p;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+      o[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+    }
+  }
+};
+
 DEV_INLINE float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 DEV_INLINE float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
