@@ -70,6 +70,23 @@ __global__ void relu_squared_kernel(T* __restrict__ out,
   }
 }
 
+template <typename T>
+__global__ void relu_squared_vec_kernel(T* __restrict__ out,
+                                        const T* __restrict__ x, int64_t nvec) {
+  constexpr int N = Vec16<T>::N;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nvec) {
+    float v[N];
+    Vec16<T>::load(x + i * N, v);
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+      const float r = fmaxf(v[e], 0.f);
+      v[e] = r * r;
+    }
+    Vec16<T>::store(out + i * N, v);
+  }
+}
+
 }  // namespace
 
 void add_layernorm(torch::Tensor out, c10::optional<torch::Tensor> branch,
@@ -126,6 +143,18 @@ void relu_squared(torch::Tensor out, torch::Tensor x) {
               out.scalar_type() == x.scalar_type() && out.numel() == x.numel());
   const int64_t n = x.numel();
   if (n == 0) return;
+  const int64_t vn = 16 / x.element_size();
+  if (n % vn == 0 && ((size_t)x.data_ptr()) % 16 == 0 &&
+      ((size_t)out.data_ptr()) % 16 == 0) {
+    const int64_t nvec = n / vn;
+    SEQ_DISPATCH_ACT(x, {
+      hipLaunchKernelGGL((relu_squared_vec_kernel<act_t>), dim3((nvec + 255) / 256),
+                         dim3(256), 0, SEQ_STREAM(), (act_t*)out.data_ptr(),
+                         (const act_t*)x.data_ptr(), nvec);
+    });
+    SEQ_CHECK_LAUNCH();
+    return;
+  }
   SEQ_DISPATCH_ACT(x, {
     hipLaunchKernelGGL((relu_squared_kernel<act_t>), dim3((n + 255) / 256),
                        dim3(256), 0, SEQ_STREAM(), (act_t*)out.data_ptr(),

@@ -47,6 +47,9 @@ DEV_INLINE void cvt4(const ushort4& v, float* o) {
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
   static constexpr int N = 4;
+  static DEV_INLINE void store(float* p, const float* o) {
+    *(float4*)p = make_float4(o[0], o[1], o[2], o[3]);
+  }
   static DEV_INLINE void load(const float* p, float* o) {
     const float4 v = *(const float4*)p;
     o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
@@ -54,6 +57,14 @@ template <> struct Vec16<float> {
 };
 template <> struct Vec16<bf16raw> {
   static constexpr int N = 8;
+  static DEV_INLINE void store(bf16raw* p, const float* o) {
+    uint4 v;
+    v.x = (uint32_t)f32_to_bf16(o[0]) | ((uint32_t)f32_to_bf16(o[1]) << 16);
+    v.y = (uint32_t)f32_to_bf16(o[2]) | ((uint32_t)f32_to_bf16(o[3]) << 16);
+    v.z = (uint32_t)f32_to_bf16(o[4]) | ((uint32_t)f32_to_bf16(o[5]) << 16);
+    v.w = (uint32_t)f32_to_bf16(o[6]) | ((uint32_t)f32_to_bf16(o[7]) << 16);
+    *(uint4*)p = v;
+  }
   static DEV_INLINE void load(const bf16raw* p, float* o) {
     const uint4 v = *(const uint4*)p;
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};

@@ -74,18 +74,19 @@ def test_gated_rmsnorm(dtype, groups, act):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_relu_squared(dtype):
-    x = torch.randn(33, 70).to(dtype)
+@pytest.mark.parametrize("cols", [70, 71 * 8])
+def test_relu_squared(dtype, cols):
+    x = torch.randn(33, cols).to(dtype)
     torch.testing.assert_close(sops.relu_squared(x.cuda()).cpu().float(),
                                sops.relu_squared(x).float(), **_tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("taps,residual", [(4, True), (3, False), (2, False), (7, True)])
-def test_causal_conv(dtype, taps, residual):
+@pytest.mark.parametrize("C", [72, 70])  # 16-byte and scalar access paths
+def test_causal_conv(dtype, taps, residual, C):
     torch.manual_seed(2)
     _, T = _meta("cpu")
-    C = 72
     wide = torch.randn(T, C + 8).to(dtype)
     w = torch.randn(C, taps)
     tails = torch.randn(6, taps - 1, C)
