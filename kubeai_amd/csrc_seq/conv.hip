@@ -40,49 +40,6 @@ __global__ void causal_conv_kernel(
   stf(y + (size_t)t * C + c, acc);
 }
 
-// The same with 16-byte accesses: a thread owns N consecutive channels of
-// one token (C a multiple of N, rows 16-byte aligned).
-template <typename T>
-__global__ void causal_conv_vec_kernel(
-    T* __restrict__ y, const T* __restrict__ x, int64_t x_stride,
-    const float* __restrict__ w, const float* __restrict__ tails,
-    const int* __restrict__ start_loc, const int* __restrict__ slots,
-    const int* __restrict__ token_seq, const int* __restrict__ positions,
-    int C, int taps, int residual) {
-  constexpr int N = Vec16<T>::N;
-  const int t = blockIdx.x;
-  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * N;
-  if (c >= C) return;
-  const int s = token_seq[t], s0 = start_loc[s], slot = slots[s];
-  const int p = positions[t], p0 = positions[s0];
-  const int K1 = taps - 1;
-  float acc[N];
-  if (residual) {
-    Vec16<T>::load(x + (size_t)t * x_stride + c, acc);
-  } else {
-#pragma unroll
-    for (int e = 0; e < N; ++e) acc[e] = 0.f;
-  }
-  for (int j = 0; j < taps; ++j) {
-    const int d = K1 - j;
-    const int sp = p - d;
-    if (sp < 0) continue;
-    float v[N];
-    if (t - d >= s0) {
-      Vec16<T>::load(x + (size_t)(t - d) * x_stride + c, v);
-    } else if (slot >= 0) {
-      const float* tp = tails + ((size_t)slot * K1 + (sp - (p0 - K1))) * C + c;
-#pragma unroll
-      for (int e = 0; e < N; e += 4) Vec16<float>::load(tp + e, v + e);
-    } else {
-      continue;
-    }
-#pragma unroll
-    for (int e = 0; e < N; ++e) acc[e] += w[(size_t)(c + e) * taps + j] * v[e];
-  }
-  Vec16<T>::store(y + (size_t)t * C + c, acc);
-}
-
 // grid (n_seq, ceil(C / 256)): advance a run's tail past its tokens. One
 // thread owns a channel's whole tail, so old rows are read before any write.
 template <typename T>
@@ -164,24 +121,6 @@ void causal_conv(torch::Tensor y, torch::Tensor x, torch::Tensor w,
               start_loc.numel() == slots.numel() + 1);
   TORCH_CHECK((C + 255) / 256 <= 65535);
   if (T == 0) return;
-  const size_t esz = x.element_size();
-  const int vn = (int)(16 / esz);
-  if (C % vn == 0 && x.stride(0) % vn == 0 && ((size_t)x.data_ptr()) % 16 == 0 &&
-      ((size_t)y.data_ptr()) % 16 == 0 && ((size_t)tails.data_ptr()) % 16 == 0) {
-    const int nthr = C / vn;
-    SEQ_DISPATCH_ACT(x, {
-      hipLaunchKernelGGL((causal_conv_vec_kernel<act_t>), dim3(T, (nthr + 255) / 256),
-                         dim3(256), 0, SEQ_STREAM(), (act_t*)y.data_ptr(),
-                         (const act_t*)x.data_ptr(), x.stride(0),
-                         (const float*)w.data_ptr(), (const float*)tails.data_ptr(),
-                         (const int*)start_loc.data_ptr(), (const int*)slots.data_ptr(),
-                         (const int*)token_seq.data_ptr(),
-                         (const int*)positions.data_ptr(), C, taps, residual ? 1 : 0);
-    });
-    SEQ_CHECK_LAUNCH();
-    launch_tail_update(tails, x, start_loc, slots, positions, C, taps - 1);
-    return;
-  }
   SEQ_DISPATCH_ACT(x, {
     hipLaunchKernelGGL((causal_conv_kernel<act_t>), dim3(T, (C + 255) / 256),
                        dim3(256), 0, SEQ_STREAM(), (act_t*)y.data_ptr(),

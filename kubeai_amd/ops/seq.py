@@ -16,7 +16,7 @@ sequence's *state slot* (engine/statecache.py). Conventions:
     gates of a recurrence, norms and attention scores are fp32 inside.
 
 Dispatch follows kubeai_amd.ops: CPU tensors run the torch references below
-(also the numerics contract of the kernels); GPU tensors require the
+(also the numerics reference of the kernels); GPU tensors require the
 ``kubeai_amd._C_seq`` HIP extension and fail loudly without it.
 """
 from __future__ import annotations
