@@ -36,7 +36,8 @@ class SyntheticTokenizer:
         return o - 29
 
     def encode(self, text: str, add_bos: bool = False) -> list[int]:
-        toks: list[int] = [self.bos_token_id] if add_bos else []
+        # a model without a begin-of-sequence token says so with a negative id
+        toks: list[int] = [self.bos_token_id] if add_bos and self.bos_token_id >= 0 else []
         span = self.vocab_size - self._lo
         for word in text.split():
             if word == "<image>" and self.image_token_id is not None:
@@ -150,7 +151,8 @@ def apply_chat_template(tokenizer, messages: list[dict]) -> list[int]:
         except Exception:
             pass
     role_ids = {"system": 3, "user": 4, "assistant": 5, "tool": 6}
-    toks: list[int] = [tokenizer.bos_token_id]
+    bos = tokenizer.bos_token_id
+    toks: list[int] = [bos] if bos is not None and bos >= 0 else []
     for m in messages:
         toks.append(role_ids.get(m.get("role", "user"), 4))
         toks.extend(tokenizer.encode(text_of(m)))

@@ -477,3 +477,33 @@ def test_state_slots_survive_preemption_and_abort(tmp_path):
             row = logits[len(prompts[rid]) - 1 + i]
             assert row[tok] >= row.max() - 1e-3 * row.std()
     assert eng.state_manager.num_free == 3
+
+
+def test_served_over_http_with_sampling():
+    """The family behind the engine's OpenAI server: greedy and sampled
+    completions through the same scheduler, sampler and tokenizer plumbing."""
+    from fastapi.testclient import TestClient
+
+    from kubeai_amd.engine.server import EngineServer, build_app
+
+    cfg = EngineConfig(model="dulotar-tiny", device="cpu", num_gpu_blocks=64,
+                       max_model_len=256, max_num_seqs=4)
+    server = EngineServer(cfg, "hybrid")
+    server.start()
+    server._ready.wait(timeout=60)
+    try:
+        with TestClient(build_app(server)) as c:
+            r = c.post("/v1/completions", json={"model": "hybrid", "prompt": "a b c d e",
+                                                "max_tokens": 6, "temperature": 0})
+            assert r.status_code == 200, r.text
+            greedy = r.json()
+            assert greedy["usage"]["completion_tokens"] >= 1
+            r2 = c.post("/v1/completions", json={"model": "hybrid", "prompt": "a b c d e",
+                                                 "max_tokens": 6, "temperature": 0})
+            assert r2.json()["choices"][0]["text"] == greedy["choices"][0]["text"]
+            r3 = c.post("/v1/completions", json={"model": "hybrid", "prompt": "a b c d e",
+                                                 "max_tokens": 6, "temperature": 0.9,
+                                                 "top_p": 0.9, "seed": 3})
+            assert r3.status_code == 200, r3.text
+    finally:
+        server.stop()
