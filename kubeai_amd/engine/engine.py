@@ -269,7 +269,8 @@ class LLMEngine:
         self.scheduler.finish_fixed(out, ended)
         for req in ended:
             self.runner.release_request(req.request_id)
-        return [rows[rid] for rid, _, _ in entries]
+        none = torch.empty((0, self.arch.vocab_size), dtype=torch.float32)
+        return [rows.get(rid, none) for rid, _, _ in entries]
 
     # ------------------------------------------------------------------
     def embed(self, tok_lists: list[list[int]]) -> list[list[float]]:

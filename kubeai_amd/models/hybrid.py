@@ -107,6 +107,8 @@ class DulotarForCausalLM(nn.Module):
                 self.embed_tokens = nn.Embedding(cfg.vocab_size, W)
                 own = {}
                 for i, spec in enumerate(hs.layers):
+                    if not 0 <= spec.weights_of < len(hs.layers):
+                        raise ValueError(f"layer {i}: weights_of out of range")
                     if spec.weights_of == i:
                         own[i] = HybridLayer(spec, W, hs.norm_eps, hs.canon_taps)
                 self.layers = nn.ModuleDict({str(i): m for i, m in own.items()})
@@ -119,7 +121,16 @@ class DulotarForCausalLM(nn.Module):
             torch.set_default_dtype(prev_dtype)
         # layer runs in execution order: a layer that uses another's tensors
         # runs that module with its own state / cache index
-        self.runs = [self.layers[str(s.weights_of)] for s in hs.layers]
+        def owner(i: int) -> int:
+            seen = set()
+            while hs.layers[i].weights_of != i:  # a shared layer may itself share
+                if i in seen:
+                    raise ValueError("weights_of forms a cycle")
+                seen.add(i)
+                i = hs.layers[i].weights_of
+            return i
+
+        self.runs = [self.layers[str(owner(i))] for i in range(len(hs.layers))]
         self.capture_layers = None  # set to a list to record per-layer residuals
 
     # -- what the runner allocates per layer run -------------------------
