@@ -57,7 +57,9 @@ class CausalConvTails(nn.Module):
 
 
 class MinGRUMixer(nn.Module):
-    """minGRU: elementwise recurrent state; gate and candidate depend on the input at t alone."""
+    """minGRU: elementwise recurrent state whose gate and candidate are
+    functions of the input at t alone, which is what lets a run be scanned
+    segment-parallel."""
 
     def __init__(self, width: int, n: int):
         super().__init__()
@@ -214,8 +216,8 @@ class LightningAttention(nn.Module):
 
 
 class ParallelMixer(nn.Module):
-    """Chunked softmax attention and lightning attention fed by one input, the
-    same input, summed with fixed scales. Both input projections are one
+    """Chunked softmax attention and lightning attention fed by one input
+    and summed with fixed scales. Both input projections are one
     GEMM; both output projections are one GEMM over the concatenated
     (pre-scaled) branch outputs."""
 

@@ -42,7 +42,8 @@ def silu(x):
 
 
 def mingru(h, W, p):
-    """minGRU: elementwise state; gate and candidate depend on the input at t alone."""
+    """minGRU: elementwise state, gate and candidate depend on the input at t alone
+    (no path from the state into the gates)."""
     z = torch.sigmoid(h @ W[p + "z"].T + W[p + "z.b"])
     u = h @ W[p + "x"].T + W[p + "x.b"]
     cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
