@@ -1,6 +1,8 @@
-// Rotary on interleaved pairs fused with the paged cache write, and softmax
-// attention of every packed token over its own sequence's cached keys under
-// a chunk / window mask, with separate key and value sizes.
+// Rotary (interleaved pairs, or split halves after a whole-row RMS norm of q
+// and k) fused with the paged cache write, and softmax attention of every
+// packed token over its own sequence's cached keys under a chunk / window
+// mask, with separate key and value sizes and an optional sink (a key of
+// score 0 without a value: one more term in the denominator).
 #include "seq_common.h"
 
 namespace {
@@ -57,6 +59,79 @@ __global__ void rope_pairs_cache_kernel(
   }
 }
 
+// grid (T). q and k rows are RMS-normed as a whole (all heads at once, plain
+// weights), then the first 2 * half dims of every head rotate with dimension
+// i paired with i + half; the rest pass. q is rewritten in place, k goes to
+// the key cache, v is copied to the value cache. fp32 throughout.
+template <typename T>
+__global__ __launch_bounds__(256) void qknorm_rope_half_cache_kernel(
+    T* __restrict__ q, int64_t q_stride, const T* __restrict__ k,
+    int64_t k_stride, const T* __restrict__ v, int64_t v_stride,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const int* __restrict__ positions, const float* __restrict__ inv_freq,
+    int half, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int64_t* __restrict__ slot_mapping, int H, int G, int D, int Dv,
+    int bs) {
+  __shared__ float red0[16], red1[16];
+  const int t = blockIdx.x;
+  const float pos = (float)positions[t];
+  const int64_t slot = slot_mapping[t];
+  T* qr = q + (size_t)t * q_stride;
+  const T* kr = k + (size_t)t * k_stride;
+  float rq = 1.f, rk = 1.f;
+  if (qw != nullptr) {
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < H * D; i += blockDim.x) {
+      const float x = ldf(qr + i);
+      sq += x * x;
+    }
+    for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
+      const float x = ldf(kr + i);
+      sk += x * x;
+    }
+    rq = 1.0f / sqrtf(block_sum(sq, red0) / (float)(H * D) + eps);
+    rk = 1.0f / sqrtf(block_sum(sk, red1) / (float)(G * D) + eps);
+  }
+  const int upr = D - half;  // units per head: `half` pairs, then single dims
+  const int nq = H * upr, nk = G * upr, nv = G * Dv;
+  const int64_t blk = slot >= 0 ? slot / bs : 0;
+  const int off = slot >= 0 ? (int)(slot % bs) : 0;
+  for (int u = threadIdx.x; u < nq + nk + nv; u += blockDim.x) {
+    if (u < nq + nk) {
+      const bool is_q = u < nq;
+      const int uu = is_q ? u : u - nq;
+      const int hd = uu / upr, i = uu % upr;
+      if (!is_q && slot < 0) continue;
+      const T* src = is_q ? qr + hd * D : kr + hd * D;
+      const float* w = is_q ? qw : kw;
+      const float r = is_q ? rq : rk;
+      T* dst = is_q ? qr + hd * D
+                    : k_cache + (((size_t)blk * G + hd) * bs + off) * D;
+      if (i < half) {
+        float a = ldf(src + i) * r, b = ldf(src + i + half) * r;
+        if (w != nullptr) {
+          a *= w[hd * D + i];
+          b *= w[hd * D + i + half];
+        }
+        float sn, cs;
+        sincosf(pos * inv_freq[i], &sn, &cs);
+        stf(dst + i, a * cs - b * sn);
+        stf(dst + i + half, b * cs + a * sn);
+      } else {
+        const int d = i + half;
+        float a = ldf(src + d) * r;
+        if (w != nullptr) a *= w[hd * D + d];
+        stf(dst + d, a);
+      }
+    } else if (slot >= 0) {
+      const int e = u - nq - nk;
+      const int g = e / Dv, d = e % Dv;
+      v_cache[(((size_t)blk * G + g) * bs + off) * Dv + d] =
+          v[(size_t)t * v_stride + g * Dv + d];
+    }
+  }
+}
+
 constexpr int kMaxDvPerLane = 8;  // value size <= 512
 
 constexpr int kDecWaves = 4;
@@ -80,7 +155,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
     const T* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ token_seq,
     const int* __restrict__ positions, float scale, float softcap, int chunk,
-    int window, float out_scale, int H, int G, int D, int Dv, int bs) {
+    int window, float out_scale, int sink, int H, int G, int D, int Dv, int bs) {
   constexpr int N = Vec16<T>::N;
   const int lpr = kVec ? Dv / N : 1;          // lanes per value row
   const int ngrp = kVec ? WAVE / lpr : 1;     // key groups of a wave
@@ -194,6 +269,7 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
     wsc[w] = mw == -INFINITY ? 0.f : expf(mw - mx);  // a wave may have had no tile
     lsum += stat[2 * w + 1] * wsc[w];
   }
+  if (sink) lsum += expf(-mx);
   const float inv = out_scale / lsum;
   for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
     float a = 0.f;
@@ -226,8 +302,8 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
     const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
     int max_blocks, const int* __restrict__ start_loc,
     const int* __restrict__ positions, int tiles_per_run, float scale,
-    float softcap, int chunk, int window, float out_scale, int H, int G, int D,
-    int Dv, int bs) {
+    float softcap, int chunk, int window, float out_scale, int sink, int H, int G,
+    int D, int Dv, int bs) {
   const int s = blockIdx.x / tiles_per_run, tile = blockIdx.x % tiles_per_run;
   const int h = blockIdx.y, g = h / (H / G);
   const int s0 = start_loc[s], s1 = start_loc[s + 1];
@@ -312,6 +388,7 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
   }
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
+  if (sink) l += expf(-m);
   if (q_ok) {
     const float inv = out_scale / l;
     bf16raw* op = out + (size_t)tq * out_stride + h * Dv + grp * 4;
@@ -372,12 +449,60 @@ void rope_pairs_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
   SEQ_CHECK_LAUNCH();
 }
 
+void qknorm_rope_half_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                c10::optional<torch::Tensor> q_weight,
+                                c10::optional<torch::Tensor> k_weight, double eps,
+                                torch::Tensor positions, torch::Tensor inv_freq,
+                                torch::Tensor k_cache, torch::Tensor v_cache,
+                                torch::Tensor slot_mapping) {
+  check_i32(positions, "positions");
+  check_f32(inv_freq, "inv_freq");
+  TORCH_CHECK(dense_heads3(q) && dense_heads3(k) && dense_heads3(v));
+  TORCH_CHECK(slot_mapping.scalar_type() == torch::kInt64 &&
+              slot_mapping.is_contiguous());
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  const int G = k.size(1), Dv = v.size(2), half = inv_freq.numel();
+  TORCH_CHECK(2 * half <= D, "rotated dims exceed the key size");
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && k.size(2) == D && v.size(1) == G);
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  TORCH_CHECK(q_weight.has_value() == k_weight.has_value());
+  if (q_weight.has_value()) {
+    check_f32(*q_weight, "q_weight");
+    check_f32(*k_weight, "k_weight");
+    TORCH_CHECK(q_weight->numel() == (int64_t)H * D && k_weight->numel() == (int64_t)G * D);
+  }
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4);
+  TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D && v_cache.size(1) == G &&
+              v_cache.size(3) == Dv && v_cache.size(2) == k_cache.size(2) &&
+              v_cache.size(0) == k_cache.size(0));
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type() &&
+              k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type());
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(q, {
+    hipLaunchKernelGGL((qknorm_rope_half_cache_kernel<act_t>), dim3(T), dim3(256), 0,
+                       SEQ_STREAM(), (act_t*)q.data_ptr(), q.stride(0),
+                       (const act_t*)k.data_ptr(), k.stride(0),
+                       (const act_t*)v.data_ptr(), v.stride(0),
+                       q_weight.has_value() ? (const float*)q_weight->data_ptr() : nullptr,
+                       k_weight.has_value() ? (const float*)k_weight->data_ptr() : nullptr,
+                       (float)eps, (const int*)positions.data_ptr(),
+                       (const float*)inv_freq.data_ptr(), half,
+                       (act_t*)k_cache.data_ptr(), (act_t*)v_cache.data_ptr(),
+                       (const int64_t*)slot_mapping.data_ptr(), H, G, D, Dv,
+                       (int)k_cache.size(2));
+  });
+  SEQ_CHECK_LAUNCH();
+}
+
 void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor k_cache, torch::Tensor v_cache,
                             torch::Tensor block_tables, torch::Tensor start_loc,
                             torch::Tensor token_seq, torch::Tensor positions,
                             int64_t max_len, double scale, double softcap,
-                            int64_t chunk, int64_t window, double out_scale) {
+                            int64_t chunk, int64_t window, double out_scale,
+                            bool sink) {
   check_i32(start_loc, "start_loc");
   check_i32(block_tables, "block_tables");
   check_i32(token_seq, "token_seq");
@@ -415,8 +540,8 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                        (const int*)block_tables.data_ptr(),
                        (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
                        (const int*)positions.data_ptr(), tiles, (float)scale,
-                       (float)softcap, (int)chunk, (int)window, (float)out_scale, H,
-                       G, D, Dv, bs);
+                       (float)softcap, (int)chunk, (int)window, (float)out_scale,
+                       (int)sink, H, G, D, Dv, bs);
     SEQ_CHECK_LAUNCH();
     return;
   }
@@ -440,7 +565,7 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (int)block_tables.size(1), (const int*)token_seq.data_ptr(),
                          (const int*)positions.data_ptr(), (float)scale,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                         H, G, D, Dv, bs);
+                         (int)sink, H, G, D, Dv, bs);
     };
     if (vec) launch(masked_paged_attention_kernel<act_t, true>);
     else launch(masked_paged_attention_kernel<act_t, false>);

@@ -34,7 +34,24 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                             torch::Tensor block_tables, torch::Tensor start_loc,
                             torch::Tensor token_seq, torch::Tensor positions,
                             int64_t max_len, double scale, double softcap,
-                            int64_t chunk, int64_t window, double out_scale);
+                            int64_t chunk, int64_t window, double out_scale,
+                            bool sink);
+void qknorm_rope_half_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                c10::optional<torch::Tensor> q_weight,
+                                c10::optional<torch::Tensor> k_weight, double eps,
+                                torch::Tensor positions, torch::Tensor inv_freq,
+                                torch::Tensor k_cache, torch::Tensor v_cache,
+                                torch::Tensor slot_mapping);
+void sandwich_rmsnorm(torch::Tensor out, c10::optional<torch::Tensor> branch,
+                      c10::optional<torch::Tensor> post_weight,
+                      torch::Tensor residual, torch::Tensor pre_weight, double eps);
+void rmsnorm_to_cache(torch::Tensor cache, torch::Tensor x, torch::Tensor weight,
+                      torch::Tensor slot_mapping, double eps);
+void sigmoid_gate(torch::Tensor out, torch::Tensor x, torch::Tensor gate);
+void router_topk(torch::Tensor logits, torch::Tensor dense, torch::Tensor weights,
+                 torch::Tensor index);
+void relu_squared_weighted(torch::Tensor out, torch::Tensor u, torch::Tensor w,
+                           int64_t group);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("add_layernorm", &add_layernorm, "fp32 residual add + LayerNorm");
@@ -47,5 +64,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rope_pairs_and_cache", &rope_pairs_and_cache,
         "interleaved-pair rotary + paged cache write");
   m.def("masked_paged_attention", &masked_paged_attention,
-        "chunk/window-masked paged softmax attention");
+        "chunk/window-masked paged softmax attention, optional sink");
+  m.def("qknorm_rope_half_and_cache", &qknorm_rope_half_and_cache,
+        "whole-row q/k RMS norm + split-half rotary + paged cache write");
+  m.def("sandwich_rmsnorm", &sandwich_rmsnorm,
+        "post-norm of a branch + fp32 residual add + next pre-norm");
+  m.def("rmsnorm_to_cache", &rmsnorm_to_cache, "RMS norm written into a paged cache");
+  m.def("sigmoid_gate", &sigmoid_gate, "x * sigmoid(gate)");
+  m.def("router_topk", &router_topk, "top-k routing with softmax over the chosen");
+  m.def("relu_squared_weighted", &relu_squared_weighted,
+        "relu(u)^2 times a per-row, per-group weight");
 }

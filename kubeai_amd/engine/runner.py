@@ -45,7 +45,7 @@ class _DecodeGraph:
         # rows' state slots are one more refreshed input (-1 on pad rows)
         self.state_slots = None
         seq = None
-        if runner.has_seq_state:
+        if runner.uses_seq_meta:
             from kubeai_amd.ops.seq import SeqMeta
 
             self.state_slots = torch.full((b_pad,), -1, dtype=torch.int32, device=dev)
@@ -150,6 +150,11 @@ class ModelRunner:
         if tp_group is not None:
             from kubeai_amd.parallel.tp import TPLlamaForCausalLM
 
+            if arch.hybrid is not None:
+                raise NotImplementedError(
+                    "tensor parallelism is not implemented for the "
+                    f"{arch.architecture} layer stack"
+                )
             if arch.post_norms:
                 raise NotImplementedError(
                     "tensor parallelism is not implemented for the gemma2 "
@@ -168,6 +173,11 @@ class ModelRunner:
         # models with per-sequence recurrent state get a slot per live
         # sequence (engine/statecache.py) and a SeqMeta in every batch
         self.has_seq_state = bool(getattr(self.model, "has_seq_state", False))
+        # kernels that take the packed runs (ops.seq.SeqMeta) need fb.seq even
+        # when the model keeps no state slots
+        self.uses_seq_meta = self.has_seq_state or bool(
+            getattr(self.model, "uses_seq_meta", False)
+        )
         if self.has_seq_state and tp_group is not None:
             raise NotImplementedError(
                 "tensor parallelism is not implemented for models with "
@@ -426,7 +436,7 @@ class ModelRunner:
         n_prefill = len(pre_lens)
         seq = None
         pos_t = t32(positions)
-        if self.has_seq_state:
+        if self.uses_seq_meta:
             from kubeai_amd.ops.seq import SeqMeta
 
             seq = SeqMeta.build(
@@ -515,7 +525,7 @@ class ModelRunner:
                 torch.tensor(
                     [ss.req.state_slot for ss in out.decode], dtype=torch.int32
                 )
-                if self.has_seq_state
+                if self.uses_seq_meta
                 else None
             ),
         )

@@ -79,6 +79,8 @@ class ModelArchConfig:
             cfg = json.load(f)
         if cfg.get("architecture") == "Dulotar":
             return dulotar_arch_config(cfg)
+        if cfg.get("architecture") == "Nugopel":
+            return nugopel_arch_config(cfg)
         hidden = cfg["hidden_size"]
         n_heads = cfg["num_attention_heads"]
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
@@ -226,6 +228,35 @@ def dulotar_arch_config(cfg: dict) -> ModelArchConfig:
             norm_eps=float(cfg["norm"]["eps"]),
             embedding_scale=float(cfg["embedding"]["scale"]),
             canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+        ),
+    )
+
+
+def nugopel_arch_config(cfg: dict) -> ModelArchConfig:
+    """Nugopel config.json -> arch config: the list of layers (mixer type,
+    the mixer's sizes and constants, the feed-forward) and the norm epsilon,
+    all as the file gives them."""
+    layers = [
+        HybridLayerSpec(type=L["type"], mixer=L["mixer"], mlp=L.get("mlp"), weights_of=i)
+        for i, L in enumerate(cfg["layers"])
+    ]
+    return ModelArchConfig(
+        architecture="nugopel",
+        vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]),
+        num_hidden_layers=len(layers),
+        intermediate_size=0,
+        num_attention_heads=0,
+        num_key_value_heads=0,
+        head_dim=0,
+        max_position_embeddings=1 << 30,  # positions are computed, not tabulated
+        bos_token_id=-1,
+        eos_token_id=-1,  # the design defines no end token
+        hybrid=HybridSpec(
+            layers=layers,
+            norm_eps=float(cfg["norm"]["eps"]),
+            embedding_scale=1.0,
+            canon_taps=0,
         ),
     )
 

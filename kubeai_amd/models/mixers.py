@@ -262,3 +262,189 @@ class SquaredReluMLP(nn.Module):
 
     def forward(self, h):
         return self.down(sops.relu_squared(self.up(h)))
+
+
+def scaled_rotary_frequencies(dims: int, base: float, scaling: dict | None):
+    """fp32 [dims/2] rotary frequencies base^(-2i/dims), optionally rescaled
+    by wavelength (scaling = {factor, low, high, original}): wavelengths
+    below original/high keep their frequency, those above original/low are
+    divided by factor, and the band between is interpolated linearly in
+    original/wavelength."""
+    import math
+
+    out = []
+    for i in range(int(dims) // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high = (float(scaling[k]) for k in ("factor", "low", "high"))
+            orig = float(scaling["original"])
+            lam = 2.0 * math.pi / f
+            if lam > orig / low:
+                f = f / factor
+            elif lam >= orig / high:
+                s = (orig / lam - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float32)
+
+
+class SinkWindowAttention(nn.Module):
+    """Softmax attention over a sliding window of cached keys with grouped
+    key/value heads and separate key and value sizes. Options, each a
+    constructor argument: an RMS norm over the whole q and the whole k
+    projection (all heads at once) before rotation, rotary on the leading
+    dims of every head in the split-half pairing with wavelength-dependent
+    frequency scaling, and a sink (a value-less key of score 0)."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, window=0,
+                 sink=False, qk_norm=False, rot_dims=0, rot_base=10000.0,
+                 rot_scaling=None, eps=1e-5):
+        super().__init__()
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.sink, self.eps = float(scale), int(window or 0), bool(sink), eps
+        self.sizes = (heads * dim, kv_heads * dim, kv_heads * vdim)
+        self.in_proj = Proj(width, sum(self.sizes))  # q | k | v
+        self.o_proj = Proj(heads * vdim, width)
+        self.q_norm = self.k_norm = None
+        if qk_norm:
+            self.q_norm, self.k_norm = _f32(heads * dim), _f32(kv_heads * dim)
+            nn.init.ones_(self.q_norm)
+            nn.init.ones_(self.k_norm)
+        self.register_buffer(
+            "inv_freq", scaled_rotary_frequencies(rot_dims, rot_base, rot_scaling),
+            persistent=False)
+
+    def state_spec(self):
+        return {}
+
+    def kv_spec(self):
+        return (self.kv_heads, self.dim, self.vdim)
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        nq, nk, nv = self.sizes
+        qkv = self.in_proj(h)
+        q = qkv[:, :nq].unflatten(-1, (self.heads, self.dim))
+        k = qkv[:, nq : nq + nk].unflatten(-1, (self.kv_heads, self.dim))
+        v = qkv[:, nq + nk :].unflatten(-1, (self.kv_heads, self.vdim))
+        k_cache, v_cache = kv_cache
+        sops.qknorm_rope_half_and_cache(q, k, v, self.q_norm, self.k_norm, self.eps,
+                                        fb.positions, self.inv_freq, k_cache, v_cache,
+                                        fb.slot_mapping)
+        out = torch.empty((T, self.heads, self.vdim), dtype=h.dtype, device=h.device)
+        sops.masked_paged_attention(q, k_cache, v_cache, fb.seq, self.scale, out,
+                                    window=self.window, sink=self.sink)
+        return self.o_proj(out.view(T, self.heads * self.vdim))
+
+
+class LatentAttention(nn.Module):
+    """Causal attention whose keys and values are per-head up-projections of
+    one low-rank latent per token; only the (RMS-normed) latent is cached,
+    as a one-head paged cache. No positions enter the scores. The heads'
+    concatenated output is gated by sigmoid of a projection of the input.
+
+    The kernel attends in latent space: the key up-projection is folded into
+    the query (q_h W_uk_h, one product per head), scores and the weighted sum
+    run against the cached latents, and the value up-projection is applied
+    to the result. With own_latent=False the layer has no down-projection and
+    reads the cache of another layer (bound by the model)."""
+
+    def __init__(self, width, heads, dim, vdim, kv_rank, scale, own_latent=True,
+                 eps=1e-5):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.rank = heads, dim, vdim, kv_rank
+        self.scale, self.own_latent, self.eps = float(scale), bool(own_latent), eps
+        self.sizes = (heads * dim, heads * vdim, kv_rank if own_latent else 0)
+        self.in_proj = Proj(width, sum(self.sizes))  # q | gate | latent
+        self.latent_norm = None
+        if own_latent:
+            self.latent_norm = _f32(kv_rank)
+            nn.init.ones_(self.latent_norm)
+        # per-head up-projections, stored for the folded products:
+        # uk_t [H, dim, rank] (q_h -> latent space), uv_t [H, rank, vdim]
+        self.uk_t = nn.Parameter(torch.empty(heads, dim, kv_rank), requires_grad=False)
+        self.uv_t = nn.Parameter(torch.empty(heads, kv_rank, vdim), requires_grad=False)
+        nn.init.normal_(self.uk_t, std=kv_rank ** -0.5)
+        nn.init.normal_(self.uv_t, std=kv_rank ** -0.5)
+        self.o_proj = Proj(heads * vdim, width)
+
+    def state_spec(self):
+        return {}
+
+    def kv_spec(self):
+        # one "head" of kv_rank dims; keys and values are the same rows
+        return (1, self.rank, 0) if self.own_latent else None
+
+    def forward(self, h, fb, state, kv_cache):
+        T = h.shape[0]
+        H, D, Dv, R = self.heads, self.dim, self.vdim, self.rank
+        nq, ng, _ = self.sizes
+        proj = self.in_proj(h)
+        c_cache = kv_cache[0]
+        if self.own_latent:
+            sops.rmsnorm_to_cache(proj[:, nq + ng :], self.latent_norm, self.eps,
+                                  c_cache, fb.slot_mapping)
+        q = proj[:, :nq].unflatten(-1, (H, D)).transpose(0, 1)  # [H, T, D]
+        ql = torch.bmm(q, self.uk_t).transpose(0, 1).contiguous()  # [T, H, R]
+        lat = torch.empty((T, H, R), dtype=h.dtype, device=h.device)
+        sops.masked_paged_attention(ql, c_cache, c_cache, fb.seq, self.scale, lat)
+        o = torch.bmm(lat.transpose(0, 1), self.uv_t).transpose(0, 1)  # [T, H, Dv]
+        o = o.reshape(T, H * Dv)
+        return self.o_proj(sops.sigmoid_gate(o, proj[:, nq : nq + ng]))
+
+
+class RoutedSquaredReluMoE(nn.Module):
+    """Mixture of squared-ReLU experts (down(relu(up h)^2), no biases) with
+    fp32 top-k routing, weights = softmax over the chosen logits, plus an
+    optional shared expert that every token uses.
+
+    All up-projections are one stacked matrix [E*ff + shared_ff, width] and
+    all down-projections one [width, E*ff + shared_ff]. Small steps (decode)
+    run them as two GEMMs over every expert with the routing weight (0 for
+    experts a token did not choose) folded into the activation, so the sum
+    over experts happens inside the second GEMM's fp32 accumulation and the
+    step has no data-dependent shapes. Large steps gather each expert's
+    tokens and run its slice of the stacked matrices."""
+
+    DENSE_MAX_TOKENS = 256
+
+    def __init__(self, width, experts, top, ff, shared_ff=0):
+        super().__init__()
+        self.experts, self.top, self.ff, self.shared_ff = experts, top, ff, int(shared_ff or 0)
+        n = experts * ff + self.shared_ff
+        self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32),
+                                   requires_grad=False)
+        nn.init.normal_(self.router, std=width ** -0.5)
+        self.up = Proj(width, n)
+        self.down = Proj(n, width)
+
+    def forward(self, h):
+        T = h.shape[0]
+        E, ff = self.experts, self.ff
+        logits = F.linear(h.float(), self.router)
+        dense, w, idx = sops.router_topk(logits, self.top)
+        if T <= self.DENSE_MAX_TOKENS:
+            a = sops.relu_squared_weighted(self.up(h), dense, ff)
+            return self.down(a)
+        out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
+        flat = idx.flatten().long()
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=E).tolist()
+        tok = order // self.top
+        wrow = w.flatten()[order].unsqueeze(1)
+        s = 0
+        for e in range(E):
+            n = counts[e]
+            if n == 0:
+                continue
+            rows = tok[s : s + n]
+            u = F.linear(h.index_select(0, rows), self.up.weight[e * ff : (e + 1) * ff])
+            a = sops.relu_squared_weighted(u, wrow[s : s + n], ff)
+            y = F.linear(a, self.down.weight[:, e * ff : (e + 1) * ff])
+            out.index_add_(0, rows, y.float())
+            s += n
+        if self.shared_ff:
+            u = F.linear(h, self.up.weight[E * ff :])
+            y = F.linear(sops.relu_squared(u), self.down.weight[:, E * ff :])
+            out.add_(y)
+        return out

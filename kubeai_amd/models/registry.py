@@ -15,10 +15,17 @@ def _dulotar():
     return DulotarForCausalLM
 
 
+def _nugopel():
+    from .nugopel import NugopelForCausalLM
+
+    return NugopelForCausalLM
+
+
 MODEL_REGISTRY = {
     "llama": _llama,
     "mixtral": _llama,
     "dulotar": _dulotar,
+    "nugopel": _nugopel,
 }
 
 
@@ -37,6 +44,7 @@ MODEL_EXTENSIONS = {
     "llama": ("_C",),
     "mixtral": ("_C",),
     "dulotar": ("_C_seq",),
+    "nugopel": ("_C_seq",),
 }
 
 

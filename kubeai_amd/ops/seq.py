@@ -330,18 +330,154 @@ def rope_pairs_and_cache(q, k, v, positions, inv_freq, k_cache, v_cache,
     return q
 
 
+def qknorm_rope_half_and_cache(q, k, v, q_weight, k_weight, eps: float, positions,
+                               inv_freq, k_cache, v_cache, slot_mapping):
+    """Whole-row RMS norm of q and of k (over all heads at once, plain fp32
+    weights of the row's size; None skips the norm), then rotary on the
+    first 2*len(inv_freq) dims of every head with dimension i paired with
+    i + len(inv_freq): (u, w) -> (u cos a - w sin a, w cos a + u sin a),
+    a = position * inv_freq[i] in fp32. q is rewritten in place; k and v go
+    to the paged caches at slot_mapping (slot < 0: no write)."""
+    if q.is_cuda:
+        _require_ext()
+        _C.qknorm_rope_half_and_cache(q, k, v, q_weight, k_weight, eps, positions,
+                                      inv_freq, k_cache, v_cache, slot_mapping)
+        return q
+    T, H, D = q.shape
+    G = k.shape[1]
+    half = inv_freq.numel()
+    a = positions.float().unsqueeze(-1) * inv_freq
+    c, s = torch.cos(a).unsqueeze(1), torch.sin(a).unsqueeze(1)
+
+    def prep(x, w, n):
+        xf = x.float().reshape(T, -1)
+        if w is not None:
+            xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) * w
+        xf = xf.view(T, n, D)
+        out = xf.clone()
+        u, ww = xf[..., :half], xf[..., half : 2 * half]
+        out[..., :half] = u * c - ww * s
+        out[..., half : 2 * half] = ww * c + u * s
+        return out.to(x.dtype)
+
+    q.copy_(prep(q, q_weight, H))
+    kr = prep(k, k_weight, G)
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    blk = (slot_mapping[ok] // bs).long()
+    off = (slot_mapping[ok] % bs).long()
+    k_cache[blk, :, off] = kr[ok].to(k_cache.dtype)
+    v_cache[blk, :, off] = v[ok].to(v_cache.dtype)
+    return q
+
+
+# ---------------------------------------------------------------------------
+# norms around both sides of a sublayer, cached latents, gates
+# ---------------------------------------------------------------------------
+
+def sandwich_rmsnorm(branch, post_weight, residual, pre_weight, eps: float,
+                     out_dtype):
+    """residual (fp32, in place) += branch / rms(branch) * post_weight, then
+    returns residual / rms(residual) * pre_weight in ``out_dtype``. rms(x) =
+    sqrt(mean(x^2) + eps). Weights are fp32 multipliers (a checkpoint that
+    stores them around zero adds the one when it is loaded). branch (serving
+    dtype or fp32) may be None: only the second norm runs."""
+    if residual.is_cuda:
+        _require_ext()
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        _C.sandwich_rmsnorm(out, branch, post_weight if branch is not None else None,
+                            residual, pre_weight, eps)
+        return out
+    if branch is not None:
+        b = branch.float()
+        residual.add_(b * torch.rsqrt((b * b).mean(-1, keepdim=True) + eps)
+                      * post_weight)
+    r = torch.rsqrt((residual * residual).mean(-1, keepdim=True) + eps)
+    return (residual * r * pre_weight).to(out_dtype)
+
+
+def rmsnorm_to_cache(x, weight, eps: float, cache, slot_mapping):
+    """cache row at slot_mapping[t] = x[t] / rms(x[t]) * weight (fp32 inside).
+    x [T, C] may be a strided column view; cache [blocks, 1, block, C]."""
+    if x.is_cuda:
+        _require_ext()
+        _C.rmsnorm_to_cache(cache, x, weight, slot_mapping, eps)
+        return
+    xf = x.float()
+    y = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) * weight
+    ok = slot_mapping >= 0
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping[ok].long()] = y[ok].to(cache.dtype)
+
+
+def sigmoid_gate(x, gate, out=None):
+    """x * sigmoid(gate), elementwise; gate may be a strided column view."""
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if x.is_cuda:
+        _require_ext()
+        _C.sigmoid_gate(out, x, gate)
+        return out
+    out.copy_((x.float() * torch.sigmoid(gate.float())).to(x.dtype))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# mixture-of-experts routing
+# ---------------------------------------------------------------------------
+
+def router_topk(logits, top: int):
+    """fp32 router logits [T, E] -> (dense [T, E], weights [T, top],
+    index int32 [T, top]): the `top` largest logits of every row (equal
+    logits: lower index first), weights = softmax over the chosen logits
+    only, dense = the same weights scattered to the experts' columns."""
+    T, E = logits.shape
+    if logits.is_cuda:
+        _require_ext()
+        dense = torch.empty((T, E), dtype=torch.float32, device=logits.device)
+        w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        _C.router_topk(logits.contiguous(), dense, w, idx)
+        return dense, w, idx
+    order = torch.sort(logits, dim=-1, descending=True, stable=True)
+    idx = order.indices[:, :top]
+    w = torch.softmax(order.values[:, :top], dim=-1)
+    dense = torch.zeros((T, E), dtype=torch.float32)
+    dense.scatter_(1, idx, w)
+    return dense, w, idx.to(torch.int32)
+
+
+def relu_squared_weighted(u, w, group: int):
+    """out[t, c] = relu(u[t, c])^2 * w[t, c // group]; columns past
+    w.shape[1] * group get weight 1. u [T, C]; w fp32 [T, groups]."""
+    if u.is_cuda:
+        _require_ext()
+        out = torch.empty_like(u)
+        _C.relu_squared_weighted(out, u, w, group)
+        return out
+    r = torch.relu(u.float())
+    r = r * r
+    n = w.shape[1] * group
+    r[:, :n] = (r[:, :n].view(u.shape[0], w.shape[1], group) * w.unsqueeze(-1)).view(
+        u.shape[0], n)
+    return r.to(u.dtype)
+
+
 # ---------------------------------------------------------------------------
 # masked paged attention (decode tokens and prompt portions alike)
 # ---------------------------------------------------------------------------
 
 def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
                            out, *, softcap: float = 0.0, chunk: int = 0,
-                           window: int = 0, out_scale: float = 1.0):
+                           window: int = 0, out_scale: float = 1.0,
+                           sink: bool = False):
     """Softmax attention of every packed token over its own sequence's cached
     keys. The token at position i sees j <= i with, when chunk > 0,
     floor(j / chunk) == floor(i / chunk) (position-aligned chunks) and, when
     window > 0, j > i - window. Scores are (q . k) * scale, then
-    softcap * tanh(score / softcap) if softcap > 0; all in fp32.
+    softcap * tanh(score / softcap) if softcap > 0; all in fp32. With sink,
+    the softmax has one more key of score 0 that carries no value (the
+    denominator grows by exp(0)).
     q [T, H, D] (strided ok), caches [blocks, G, block, D | Dv];
     out [T, H, Dv] may be a strided view; out = attention * out_scale."""
     if q.is_cuda:
@@ -349,7 +485,7 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         _C.masked_paged_attention(out, q, k_cache, v_cache, meta.block_tables,
                                   meta.start_loc, meta.token_seq, meta.positions,
                                   meta.max_len, scale, softcap, chunk, window,
-                                  out_scale)
+                                  out_scale, sink)
         return out
     T, H, D = q.shape
     G, bs = k_cache.shape[1], k_cache.shape[2]
@@ -382,7 +518,11 @@ def masked_paged_attention(q, k_cache, v_cache, meta: SeqMeta, scale: float,
         if window > 0:
             vis &= j.view(1, -1) > pos.view(-1, 1) - window
         s = s.masked_fill(~vis.unsqueeze(0), float("-inf"))
+        if sink:
+            s = torch.cat([s, torch.zeros_like(s[..., :1])], dim=-1)
         p = torch.softmax(s, dim=-1)
+        if sink:
+            p = p[..., :-1]
         o = torch.einsum("htl,lhd->thd", p, vs) * out_scale
         out[s0 : s0 + n] = o.to(out.dtype)
     return out
