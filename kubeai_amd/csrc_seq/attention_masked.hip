@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_half_cache_kernel(
   }
 }
 
-constexpr int kMaxDvPerLane = 8;  // value size <= 512
+constexpr int kMaxDvPerLane = 16;  // value size <= 1024
 
 constexpr int kDecWaves = 4;
 
@@ -286,8 +286,6 @@ __global__ __launch_bounds__(kDecWaves * WAVE) void masked_paged_attention_kerne
 typedef __attribute__((ext_vector_type(4))) short bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int kMaxDSteps = 8;    // key size <= 128
-constexpr int kMaxDvTiles = 16;  // value size <= 256
 
 // Prompt portions on the matrix cores (bf16, key and value sizes multiples
 // of 16). grid (n_seq * tiles_per_run, H), one wave per 16 consecutive
@@ -296,6 +294,9 @@ constexpr int kMaxDvTiles = 16;  // value size <= 256
 //   fp32 scale, cap, mask, running max / sum per query (a query is a lane
 //   column, so its statistics never leave the lane quad 16 apart)
 //   O^T += V^T P^T with P^T taken from S^T's accumulator layout as is.
+// kMaxDSteps * 16 bounds the key size and kMaxDvTiles * 16 the value size
+// (the query fragments and the output accumulators live in registers).
+template <int kMaxDSteps, int kMaxDvTiles>
 __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
     bf16raw* __restrict__ out, int64_t out_stride, const bf16raw* __restrict__ q,
     int64_t q_stride, const bf16raw* __restrict__ k_cache,
@@ -528,20 +529,23 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
     return ((size_t)t.data_ptr()) % 8 == 0 && t.stride(0) % 4 == 0;
   };
   if (q.scalar_type() == torch::kBFloat16 && max_len > 1 && D % 16 == 0 &&
-      Dv % 16 == 0 && D <= 16 * kMaxDSteps && Dv <= 16 * kMaxDvTiles && al8(q) &&
-      al8(out)) {
+      Dv % 16 == 0 && D <= 512 && Dv <= 512 && al8(q) && al8(out)) {
     // prompt portions: matrix-core kernel over 16-query tiles of every run
     const int tiles = (int)((max_len + 15) / 16);
-    hipLaunchKernelGGL(masked_prefill_mfma_kernel, dim3(n_seq * tiles, H),
-                       dim3(WAVE), 0, SEQ_STREAM(), (bf16raw*)out.data_ptr(),
-                       out.stride(0), (const bf16raw*)q.data_ptr(), q.stride(0),
-                       (const bf16raw*)k_cache.data_ptr(),
-                       (const bf16raw*)v_cache.data_ptr(),
-                       (const int*)block_tables.data_ptr(),
-                       (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
-                       (const int*)positions.data_ptr(), tiles, (float)scale,
-                       (float)softcap, (int)chunk, (int)window, (float)out_scale,
-                       (int)sink, H, G, D, Dv, bs);
+    auto launch = [&](auto kern) {
+      hipLaunchKernelGGL(kern, dim3(n_seq * tiles, H), dim3(WAVE), 0, SEQ_STREAM(),
+                         (bf16raw*)out.data_ptr(), out.stride(0),
+                         (const bf16raw*)q.data_ptr(), q.stride(0),
+                         (const bf16raw*)k_cache.data_ptr(),
+                         (const bf16raw*)v_cache.data_ptr(),
+                         (const int*)block_tables.data_ptr(),
+                         (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
+                         (const int*)positions.data_ptr(), tiles, (float)scale,
+                         (float)softcap, (int)chunk, (int)window, (float)out_scale,
+                         (int)sink, H, G, D, Dv, bs);
+    };
+    if (D <= 128 && Dv <= 256) launch(masked_prefill_mfma_kernel<8, 16>);
+    else launch(masked_prefill_mfma_kernel<32, 32>);
     SEQ_CHECK_LAUNCH();
     return;
   }

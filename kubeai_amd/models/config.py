@@ -691,6 +691,44 @@ PRESETS: dict[str, ModelArchConfig] = {
 }
 
 
+def nugopel_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
+                   window: int = 1024, kv_rank: int = 128, experts: int = 8,
+                   top: int = 2) -> ModelArchConfig:
+    """A Nugopel stack of the given size with random-init weights: the layer
+    pattern (window attention, latent attention with its own latent, window
+    attention, latent attention reading the earlier latent) repeats to the
+    requested depth; every layer has a routed feed-forward. Attention has
+    width/head_dim query heads over a quarter as many key/value heads. The
+    experts are sized so that the feed-forward work per token (chosen
+    experts + shared) is that of a dense 3.5 x width gated feed-forward."""
+    heads = max(1, width // head_dim)
+    # a gated dense layer moves 3 * width * 3.5 width weights per token; the
+    # squared-ReLU experts have two matrices: (top + 1) * ff * 2 = 10.5 width
+    ff = max(16, int(10.5 * width / (2 * (top + 1))) // 16 * 16)
+    mlp = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "top": top}, "shared": {"ff": ff}}
+    attn = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": head_dim,
+            "vdim": head_dim, "scale": head_dim ** -0.5, "mask": {"size": window},
+            "rot": {"base": 500000.0, "dims": head_dim // 2,
+                    "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                "original": 8192}}}
+    lat = {"heads": heads, "dim": head_dim, "vdim": head_dim, "kv_rank": kv_rank,
+           "scale": head_dim ** -0.5}
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append({"type": "attention", "mixer": attn, "mlp": mlp})
+        elif i % 4 == 1:
+            out.append({"type": "latent_attention", "mixer": dict(lat), "mlp": mlp})
+        else:
+            out.append({"type": "latent_attention",
+                        "mixer": dict(lat, kv_from=i - 2), "mlp": mlp})
+    return nugopel_arch_config({
+        "architecture": "Nugopel", "vocab": vocab, "width": width,
+        "norm": {"eps": 1e-5}, "layers": out,
+    })
+
+
 def dulotar_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 128,
                    chunk: int = 1024, ff_mult: int = 4) -> ModelArchConfig:
     """A Dulotar stack of the given size with random-init weights: the
@@ -723,6 +761,11 @@ def dulotar_preset(width: int, layers: int, vocab: int = 32000, head_dim: int = 
 
 
 PRESETS.update({
+    "nugopel-tiny": nugopel_preset(128, 4, vocab=512, head_dim=32, window=48,
+                                   kv_rank=64, experts=4, top=2),
+    "nugopel-1k": nugopel_preset(1024, 12),
+    "nugopel-2k": nugopel_preset(2048, 12),
+    "nugopel-4k": nugopel_preset(4096, 6),
     "dulotar-tiny": dulotar_preset(128, 3, vocab=512, head_dim=32, chunk=64),
     "dulotar-1k": dulotar_preset(1024, 12),
     "dulotar-2k": dulotar_preset(2048, 12),

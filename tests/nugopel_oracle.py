@@ -170,3 +170,62 @@ def forward(cfg, W, tokens, capture=None):
             capture.append(x.copy())
     x = norm_one_plus(x, W["final.norm"], eps)
     return x @ W["head"].T
+
+
+def random_weights(cfg, seed):
+    """{name: bfloat16 torch tensor} for a config; norm offsets around zero,
+    plain norm weights around one."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+
+    def mat(name, n_out, n_in, gain=1.0):
+        W[name] = (torch.randn(n_out, n_in, generator=g) * gain * n_in ** -0.5).bfloat16()
+
+    def vec(name, n, center):
+        W[name] = (center + 0.2 * torch.randn(n, generator=g)).bfloat16()
+
+    width, vocab = cfg["width"], cfg["vocab"]
+    W["embed"] = torch.randn(vocab, width, generator=g).bfloat16()
+    mat("head", vocab, width)
+    vec("final.norm", width, 0.0)
+    for i, L in enumerate(cfg["layers"]):
+        p, mx = f"l{i}.", L["mixer"]
+        vec(p + "norm1", width, 0.0)
+        vec(p + "norm1b", width, 0.0)
+        if L["type"] == "attention":
+            H, G, D, Dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+            mat(p + "mix.q", H * D, width)
+            mat(p + "mix.k", G * D, width)
+            mat(p + "mix.v", G * Dv, width)
+            vec(p + "mix.q.norm", H * D, 1.0)
+            vec(p + "mix.k.norm", G * D, 1.0)
+            mat(p + "mix.o", width, H * Dv)
+        else:
+            H, D, Dv, R = mx["heads"], mx["dim"], mx["vdim"], mx["kv_rank"]
+            mat(p + "mix.q", H * D, width, 2.0)
+            if mx.get("kv_from") is None:
+                mat(p + "mix.dkv", R, width)
+                vec(p + "mix.dkv.norm", R, 1.0)
+            mat(p + "mix.uk", H * D, R, 2.0)
+            mat(p + "mix.uv", H * Dv, R)
+            mat(p + "mix.g", H * Dv, width)
+            mat(p + "mix.o", width, H * Dv)
+        mlp = L.get("mlp")
+        if mlp is not None:
+            vec(p + "norm2", width, 0.0)
+            vec(p + "norm2b", width, 0.0)
+            ff = mlp["expert"]["ff"]
+            for e in range(mlp["router"]["experts"]):
+                mat(f"{p}mlp.e{e}.up", ff, width)
+                mat(f"{p}mlp.e{e}.down", width, ff)
+            mat(p + "mlp.router", mlp["router"]["experts"], width, 3.0)
+            if mlp.get("shared"):
+                mat(p + "mlp.shared.up", mlp["shared"]["ff"], width)
+                mat(p + "mlp.shared.down", width, mlp["shared"]["ff"])
+    return W
+
+
+def as_float64(W):
+    return {k: v.double().numpy() for k, v in W.items()}
