@@ -91,8 +91,11 @@ def get_args():
     )
     p.add_argument("--compare-hybrid", action="store_true",
                    help="instead of the headline workload: prefill/decode "
-                   "throughput of the Dulotar hybrid beside an equal-size Llama "
-                   "(benchmarks/hybrid_compare.py)")
+                   "throughput of a layer-list design beside the closest "
+                   "equal-size Llama-family stack (benchmarks/hybrid_compare.py)")
+    p.add_argument("--compare-design", default="dulotar",
+                   choices=["dulotar", "nugopel"],
+                   help="which design --compare-hybrid measures")
     p.add_argument("--compare-sizes", default="1k,2k,4k")
     return p.parse_args()
 

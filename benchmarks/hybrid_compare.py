@@ -1,7 +1,10 @@
-"""Prefill and decode throughput of the Dulotar hybrid beside a Llama stack
-of equal width, depth and (about) parameter count, random weights, one GPU.
+"""Prefill and decode throughput of a layer-list design (Dulotar, Nugopel)
+beside the closest homogeneous stack of equal width, depth and (about)
+parameter count, random weights, one GPU: a dense Llama for Dulotar, a
+Mixtral-style routed Llama (same number of experts and choices) for Nugopel.
 
-    python bench.py --compare-hybrid [--compare-sizes 1k,2k,4k]
+    python bench.py --compare-hybrid [--compare-design dulotar|nugopel]
+                    [--compare-sizes 1k,2k,4k]
 
 Prefill: one sequence's whole prompt as a single fixed step (both families
 go through LLMEngine.step_fixed, i.e. the packed forward without sampling).
@@ -19,8 +22,7 @@ import torch
 
 from kubeai_amd.models.config import PRESETS, ModelArchConfig
 
-SIZES = {"1k": ("dulotar-1k", 1024, 12), "2k": ("dulotar-2k", 2048, 12),
-         "4k": ("dulotar-4k", 4096, 6)}
+SIZES = {"1k": (1024, 12), "2k": (2048, 12), "4k": (4096, 6)}
 
 
 def _log(msg: str) -> None:
@@ -36,17 +38,22 @@ def _params(model) -> int:
     return n
 
 
-def _llama_like(width: int, layers: int, vocab: int, target_params: int) -> ModelArchConfig:
+def _llama_like(width: int, layers: int, vocab: int, target_params: int,
+                experts: int = 0, top: int = 2) -> ModelArchConfig:
+    """experts > 0: every feed-forward is a routed mixture of that many gated
+    experts (the Mixtral layout), sized to the same parameter count."""
     heads = width // 128
     kv = max(1, heads // 4)
     attn = width * (heads + 2 * kv) * 128 + heads * 128 * width
     fixed = 2 * vocab * width + layers * attn
-    inter = max(256, int((target_params - fixed) / (3 * width * layers)) // 256 * 256)
+    per_inter = 3 * width * layers * max(1, experts)
+    inter = max(256, int((target_params - fixed) / per_inter) // 256 * 256)
     return ModelArchConfig(
-        architecture="llama", vocab_size=vocab, hidden_size=width,
-        intermediate_size=inter, num_hidden_layers=layers, num_attention_heads=heads,
-        num_key_value_heads=kv, head_dim=128, max_position_embeddings=16384,
-        rope_theta=10000.0, eos_token_id=2, bos_token_id=1,
+        architecture="mixtral" if experts else "llama", vocab_size=vocab,
+        hidden_size=width, intermediate_size=inter, num_hidden_layers=layers,
+        num_attention_heads=heads, num_key_value_heads=kv, head_dim=128,
+        max_position_embeddings=16384, rope_theta=10000.0, eos_token_id=2,
+        bos_token_id=1, num_local_experts=experts, num_experts_per_tok=top,
     )
 
 
@@ -112,21 +119,31 @@ def main(args) -> None:
     sizes = [s for s in (args.compare_sizes or "1k,2k,4k").split(",") if s]
     prefill_lens = [2048, 8192] if device == "cuda" else [64]
     batches = [(64, 1536), (8, 3584)] if device == "cuda" else [(2, 32)]
+    design = getattr(args, "compare_design", None) or "dulotar"
+    if design not in ("dulotar", "nugopel"):
+        raise SystemExit(f"unknown design {design!r}")
     for key in sizes:
-        name, width, layers = SIZES[key]
-        if device == "cpu":
-            name = "dulotar-tiny"
+        width, layers = SIZES[key]
+        name = f"{design}-{key}" if device == "cuda" else f"{design}-tiny"
         arch = PRESETS[name]
         max_len = 8192 + 256
         blocks = (max(b * (c + 128) for b, c in batches) + max_len) // 16 + 64
-        _log(f"dulotar {key}: building engine ({name})")
+        _log(f"{design} {key}: building engine ({name})")
         eng = _engine(name, device, blocks, 64, max_len)
         n_params = _params(eng.runner.model)
         ref_name = f"llama-like-{key}"
-        PRESETS[ref_name] = _llama_like(
-            arch.hidden_size, arch.num_hidden_layers, arch.vocab_size, n_params)
-        for fam, model_name in (("dulotar", name), ("llama", ref_name)):
-            if fam == "llama":
+        ref_fam = "llama"
+        moe = arch.hybrid.layers[0].mlp if design == "nugopel" else None
+        if moe:
+            ref_fam = "mixtral"
+            PRESETS[ref_name] = _llama_like(
+                arch.hidden_size, arch.num_hidden_layers, arch.vocab_size, n_params,
+                experts=int(moe["router"]["experts"]), top=int(moe["router"]["top"]))
+        else:
+            PRESETS[ref_name] = _llama_like(
+                arch.hidden_size, arch.num_hidden_layers, arch.vocab_size, n_params)
+        for fam, model_name in ((design, name), (ref_fam, ref_name)):
+            if fam == ref_fam:
                 del eng
                 if device == "cuda":
                     torch.cuda.empty_cache()

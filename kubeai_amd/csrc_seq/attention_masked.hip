@@ -410,7 +410,9 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
 }  // namespace
 
 static bool dense_heads3(const torch::Tensor& t) {
-  return t.dim() == 3 && t.stride(2) == 1 && t.stride(1) == t.size(2);
+  // heads are addressed as row + h * size(2): a single head's stride is free
+  return t.dim() == 3 && (t.size(2) == 1 || t.stride(2) == 1) &&
+         (t.size(1) == 1 || t.stride(1) == t.size(2));
 }
 
 void rope_pairs_and_cache(torch::Tensor q, torch::Tensor k, torch::Tensor v,

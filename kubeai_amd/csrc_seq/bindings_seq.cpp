@@ -48,6 +48,8 @@ void sandwich_rmsnorm(torch::Tensor out, c10::optional<torch::Tensor> branch,
 void rmsnorm_to_cache(torch::Tensor cache, torch::Tensor x, torch::Tensor weight,
                       torch::Tensor slot_mapping, double eps);
 void sigmoid_gate(torch::Tensor out, torch::Tensor x, torch::Tensor gate);
+void head_linear(torch::Tensor y, torch::Tensor x, torch::Tensor w,
+                 c10::optional<torch::Tensor> gate);
 void router_topk(torch::Tensor logits, torch::Tensor dense, torch::Tensor weights,
                  torch::Tensor index);
 void relu_squared_weighted(torch::Tensor out, torch::Tensor u, torch::Tensor w,
@@ -71,6 +73,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "post-norm of a branch + fp32 residual add + next pre-norm");
   m.def("rmsnorm_to_cache", &rmsnorm_to_cache, "RMS norm written into a paged cache");
   m.def("sigmoid_gate", &sigmoid_gate, "x * sigmoid(gate)");
+  m.def("head_linear", &head_linear,
+        "per-head linear maps with an optional sigmoid output gate");
   m.def("router_topk", &router_topk, "top-k routing with softmax over the chosen");
   m.def("relu_squared_weighted", &relu_squared_weighted,
         "relu(u)^2 times a per-row, per-group weight");

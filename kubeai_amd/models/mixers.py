@@ -360,12 +360,13 @@ class LatentAttention(nn.Module):
         if own_latent:
             self.latent_norm = _f32(kv_rank)
             nn.init.ones_(self.latent_norm)
-        # per-head up-projections, stored for the folded products:
-        # uk_t [H, dim, rank] (q_h -> latent space), uv_t [H, rank, vdim]
-        self.uk_t = nn.Parameter(torch.empty(heads, dim, kv_rank), requires_grad=False)
-        self.uv_t = nn.Parameter(torch.empty(heads, kv_rank, vdim), requires_grad=False)
-        nn.init.normal_(self.uk_t, std=kv_rank ** -0.5)
-        nn.init.normal_(self.uv_t, std=kv_rank ** -0.5)
+        # per-head up-projections as Linear-style weights of the folded maps:
+        # uk_r [H, rank, dim] takes q_h into latent space (the transposed key
+        # up-projection), uv [H, vdim, rank] takes the attended latent out
+        self.uk_r = nn.Parameter(torch.empty(heads, kv_rank, dim), requires_grad=False)
+        self.uv = nn.Parameter(torch.empty(heads, vdim, kv_rank), requires_grad=False)
+        nn.init.normal_(self.uk_r, std=kv_rank ** -0.5)
+        nn.init.normal_(self.uv, std=kv_rank ** -0.5)
         self.o_proj = Proj(heads * vdim, width)
 
     def state_spec(self):
@@ -384,13 +385,11 @@ class LatentAttention(nn.Module):
         if self.own_latent:
             sops.rmsnorm_to_cache(proj[:, nq + ng :], self.latent_norm, self.eps,
                                   c_cache, fb.slot_mapping)
-        q = proj[:, :nq].unflatten(-1, (H, D)).transpose(0, 1)  # [H, T, D]
-        ql = torch.bmm(q, self.uk_t).transpose(0, 1).contiguous()  # [T, H, R]
+        ql = sops.head_linear(proj[:, :nq].unflatten(-1, (H, D)), self.uk_r)  # [T, H, R]
         lat = torch.empty((T, H, R), dtype=h.dtype, device=h.device)
         sops.masked_paged_attention(ql, c_cache, c_cache, fb.seq, self.scale, lat)
-        o = torch.bmm(lat.transpose(0, 1), self.uv_t).transpose(0, 1)  # [T, H, Dv]
-        o = o.reshape(T, H * Dv)
-        return self.o_proj(sops.sigmoid_gate(o, proj[:, nq : nq + ng]))
+        o = sops.head_linear(lat, self.uv, gate=proj[:, nq : nq + ng])  # [T, H, Dv]
+        return self.o_proj(o.view(T, H * Dv))
 
 
 class RoutedSquaredReluMoE(nn.Module):

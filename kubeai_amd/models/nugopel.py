@@ -197,8 +197,8 @@ class NugopelForCausalLM(nn.Module):
                     put(m.latent_norm, get(q + "dkv.norm"))
                 put(m.in_proj.weight, torch.cat(parts))
                 H, D, Dv, R = m.heads, m.dim, m.vdim, m.rank
-                put(m.uk_t, get(q + "uk").reshape(H, D, R))
-                put(m.uv_t, get(q + "uv").reshape(H, Dv, R).transpose(1, 2))
+                put(m.uk_r, get(q + "uk").reshape(H, D, R).transpose(1, 2))
+                put(m.uv, get(q + "uv").reshape(H, Dv, R))
                 put(m.o_proj.weight, get(q + "o"))
             if layer.mlp is not None:
                 put(layer.norm2, one_plus(p + "norm2"))

@@ -422,6 +422,23 @@ def sigmoid_gate(x, gate, out=None):
     return out
 
 
+def head_linear(x, w, gate=None):
+    """y[t, h, :] = w[h] @ x[t, h, :], times sigmoid(gate[t, h, :]) if a gate
+    is given. x [T, H, A] (a view with strided rows is fine), w [H, B, A],
+    gate [T, H*B] (strided rows fine) -> y [T, H, B], fp32 accumulation."""
+    T, H, _ = x.shape
+    B = w.shape[1]
+    if x.is_cuda:
+        _require_ext()
+        y = torch.empty((T, H, B), dtype=x.dtype, device=x.device)
+        _C.head_linear(y, x, w, gate)
+        return y
+    y = torch.einsum("tha,hba->thb", x.float(), w.float())
+    if gate is not None:
+        y = y * torch.sigmoid(gate.float()).reshape(T, H, B)
+    return y.to(x.dtype).contiguous()
+
+
 # ---------------------------------------------------------------------------
 # mixture-of-experts routing
 # ---------------------------------------------------------------------------
