@@ -407,6 +407,254 @@ __global__ __launch_bounds__(WAVE) void masked_prefill_mfma_kernel(
   }
 }
 
+constexpr float kLog2e = 1.4426950408889634f;
+
+// two fp32 -> packed bf16 pair (round to nearest even), low half first
+DEV_INLINE uint32_t cvt_pk_bf16(float a, float b) {
+  uint32_t r;
+  asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+constexpr int kKT = 32;      // keys staged per iteration
+constexpr int kKPad = 8;     // padding of a staged key row (elements)
+constexpr int kVPad = 4;     // padding of a staged transposed value row
+
+// Prompt portions on the matrix cores with the key / value tiles shared
+// through LDS. A block of HW * QW waves covers QW * 16 consecutive queries of
+// a run for HW query heads of one key/value head (for latent attention all
+// heads share the one cached row, for grouped heads the group does). Per
+// iteration the block stages 32 keys: K rows as they lie in the cache
+// (16-byte loads, padded rows) and V transposed ([value dim][key]), so both
+// MFMA operands are 8-byte LDS reads. Two LDS buffers: the next tile is loaded
+// into registers before the products of the current one and written to the
+// other buffer after them, one barrier per iteration. Masking and the fp32
+// softmax statistics are those of masked_prefill_mfma_kernel; P V contracts
+// all 32 keys of a tile in one v_mfma_f32_16x16x32_bf16 per 16 value dims (a
+// lane's eight contraction slots are keys grp*4 + 0..3 and 16 + grp*4 + 0..3,
+// for P and V alike), and so does K Q^T over 32 key dims when the key size
+// allows (kWideQK).
+typedef __attribute__((ext_vector_type(8))) short bf16x8;
+
+template <int kMaxDSteps, int kMaxDvTiles, bool kWideQK>
+__global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
+    bf16raw* __restrict__ out, int64_t out_stride, const bf16raw* __restrict__ q,
+    int64_t q_stride, const bf16raw* __restrict__ k_cache,
+    const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
+    int max_blocks, const int* __restrict__ start_loc,
+    const int* __restrict__ positions, int tiles_per_run, float scale,
+    float softcap, int chunk, int window, float out_scale, int sink, int H, int G,
+    int D, int Dv, int bs, int HW, int QW) {
+  extern __shared__ __attribute__((aligned(16))) bf16raw lds[];
+  constexpr int kKVec = kKT * kMaxDSteps * 16 / 8 / 256;   // per thread, 256 threads
+  constexpr int kVVec = kKT * kMaxDvTiles * 16 / 8 / 256;
+  const int nthr = blockDim.x;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int col = lane & 15, grp = lane >> 4;
+  const int hw = wave % HW, qw = wave / HW;
+  const int s = blockIdx.x / tiles_per_run, tile = blockIdx.x % tiles_per_run;
+  const int g = blockIdx.y, rep = H / G;
+  const int hz = blockIdx.z * HW + hw;
+  const int s0 = start_loc[s], s1 = start_loc[s + 1];
+  const int bq0 = s0 + tile * QW * 16;
+  if (bq0 >= s1) return;  // the whole block: no barrier is skipped
+  const int bnq = min(QW * 16, s1 - bq0);
+  const int bpos_min = positions[bq0], bpos_max = bpos_min + bnq - 1;
+  auto lower = [&](int p) {
+    int lo = 0;
+    if (chunk > 0) lo = (p / chunk) * chunk;
+    if (window > 0) lo = max(lo, p - window + 1);
+    return lo;
+  };
+  const int q0 = bq0 + qw * 16;
+  const bool wave_on = q0 < s1 && hz < rep;
+  const int nq = wave_on ? min(16, s1 - q0) : 0;
+  const int h = g * rep + min(hz, rep - 1);
+  const bool q_ok = wave_on && col < nq;
+  const int tq = wave_on ? q0 + min(col, nq - 1) : bq0;
+  const int pos_q = q_ok ? positions[tq] : -1;
+  const int wpos_min = wave_on ? positions[q0] : 0, wpos_max = wpos_min + nq - 1;
+  const int lo_q = q_ok ? lower(pos_q) : 0;
+  const int wlo = lower(wpos_min);
+  const int blo = lower(bpos_min);
+  const int* bt = block_tables + (size_t)s * max_blocks;
+  const int nks = D / 16, ndt = Dv / 16;
+  const int krow = D + kKPad, vrow = kKT + kVPad;  // LDS row lengths (elements)
+  const int buf_elems = kKT * krow + Dv * vrow;
+  const int kcpr = D / 8, vcpr = Dv / 8;  // 16-byte chunks per cached row
+
+  // query fragments: [ks] 4 dims at ks*16 + grp*4, or (wide) [kc] 8 dims at
+  // kc*32 + grp*8
+  bf16x4 qf[kWideQK ? 1 : kMaxDSteps];
+  bf16x8 qf8[kWideQK ? kMaxDSteps / 2 : 1];
+  const bf16raw* qrow = q + (size_t)tq * q_stride + h * D;
+  if (kWideQK) {
+#pragma unroll
+    for (int kc = 0; kc < kMaxDSteps / 2; ++kc)
+      if (kc < D / 32) {
+        const bf16x4 a = *(const bf16x4*)(qrow + kc * 32 + grp * 8);
+        const bf16x4 b = *(const bf16x4*)(qrow + kc * 32 + grp * 8 + 4);
+        qf8[kc] = (bf16x8){a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+      }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < kMaxDSteps; ++ks)
+      if (ks < nks) qf[ks] = *(const bf16x4*)(qrow + ks * 16 + grp * 4);
+  }
+  f32x4 oacc[kMaxDvTiles];
+#pragma unroll
+  for (int dt = 0; dt < kMaxDvTiles; ++dt) oacc[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  uint4 kreg[kKVec], vreg[kVVec];
+  // K: consecutive threads take consecutive chunks of a row (coalesced);
+  // V: consecutive threads take consecutive keys at one chunk, so that the
+  // transposed 2-byte LDS writes of a wave fall into consecutive addresses
+  auto load_tile = [&](int j0) {
+#pragma unroll
+    for (int i = 0; i < kKVec; ++i) {
+      const int v = i * nthr + threadIdx.x;
+      const int row = v / kcpr, c = v % kcpr;
+      if (row < kKT) {
+        const int j = min(j0 + row, bpos_max);
+        kreg[i] = *(const uint4*)(k_cache +
+            (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * D + c * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kVVec; ++i) {
+      const int v = i * nthr + threadIdx.x;
+      const int row = v % kKT, c = v / kKT;
+      if (c < vcpr) {
+        const int j = min(j0 + row, bpos_max);
+        vreg[i] = *(const uint4*)(v_cache +
+            (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * Dv + c * 8);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+    bf16raw* ks_ = lds + buf * buf_elems;
+    bf16raw* vs_ = ks_ + kKT * krow;
+#pragma unroll
+    for (int i = 0; i < kKVec; ++i) {
+      const int v = i * nthr + threadIdx.x;
+      const int row = v / kcpr, c = v % kcpr;
+      if (row < kKT) *(uint4*)(ks_ + row * krow + c * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kVVec; ++i) {
+      const int v = i * nthr + threadIdx.x;
+      const int row = v % kKT, c = v / kKT;
+      if (c < vcpr) {
+        const uint32_t wv[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vs_[(c * 8 + 2 * e) * vrow + row] = (bf16raw)(wv[e] & 0xffffu);
+          vs_[(c * 8 + 2 * e + 1) * vrow + row] = (bf16raw)(wv[e] >> 16);
+        }
+      }
+    }
+  };
+
+  load_tile(blo);
+  store_tile(0);
+  __syncthreads();
+  int buf = 0;
+  for (int j0 = blo; j0 <= bpos_max; j0 += kKT, buf ^= 1) {
+    const bool more = j0 + kKT <= bpos_max;
+    if (more) load_tile(j0 + kKT);
+    const bf16raw* ks_ = lds + buf * buf_elems;
+    const bf16raw* vs_ = ks_ + kKT * krow;
+    // wave-uniform: something of this tile is visible to the wave's queries
+    if (wave_on && j0 <= wpos_max && j0 + kKT - 1 >= wlo) {
+      f32x4 sacc[2];
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        sacc[sub] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        const bf16raw* kp = ks_ + (sub * 16 + col) * krow;
+        if (kWideQK) {
+#pragma unroll
+          for (int kc = 0; kc < kMaxDSteps / 2; ++kc)
+            if (kc < D / 32)
+              sacc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  *(const bf16x8*)(kp + kc * 32 + grp * 8), qf8[kc], sacc[sub], 0, 0, 0);
+        } else {
+#pragma unroll
+          for (int ks = 0; ks < kMaxDSteps; ++ks)
+            if (ks < nks)
+              sacc[sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                  *(const bf16x4*)(kp + ks * 16 + grp * 4), qf[ks], sacc[sub], 0, 0, 0);
+        }
+      }
+      // this lane: query `col`, keys j0 + sub * 16 + grp * 4 + i. Scores and
+      // the running max are kept in the base-2 domain (score * log2 e), so
+      // every exponential is one v_exp_f32.
+      float sc[8];
+      float mt = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = j0 + (e >> 2) * 16 + grp * 4 + (e & 3);
+        float x = sacc[e >> 2][e & 3] * scale;
+        if (softcap > 0.f) x = softcap * tanhf(x / softcap);
+        const bool vis = j <= pos_q && j >= lo_q;
+        sc[e] = vis ? x * kLog2e : -INFINITY;
+        mt = fmaxf(mt, sc[e]);
+      }
+      mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
+      mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
+      const float m_new = fmaxf(m, mt);
+      // no visible key so far: keep everything at zero without forming inf - inf
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = __builtin_amdgcn_exp2f(m - m_use);
+      float pv[8];
+      float ps = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);
+        ps += pv[e];
+      }
+      union { bf16x8 v; uint32_t u[4]; } pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pk.u[e] = cvt_pk_bf16(pv[2 * e], pv[2 * e + 1]);
+      const bf16x8 pb = pk.v;
+      l = l * corr + ps;
+      m = m_new;
+      const bf16raw* vp = vs_ + col * vrow + grp * 4;
+#pragma unroll
+      for (int dt = 0; dt < kMaxDvTiles; ++dt) {
+        if (dt < ndt) {
+          const bf16x4 v0 = *(const bf16x4*)(vp + dt * 16 * vrow);
+          const bf16x4 v1 = *(const bf16x4*)(vp + dt * 16 * vrow + 16);
+          const bf16x8 vf = (bf16x8){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+          f32x4 a = oacc[dt];
+          a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
+          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, a, 0, 0, 0);
+        }
+      }
+    }
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (sink) l += __builtin_amdgcn_exp2f(-m);
+  if (q_ok) {
+    const float inv = out_scale / l;
+    bf16raw* op = out + (size_t)tq * out_stride + h * Dv + grp * 4;
+#pragma unroll
+    for (int dt = 0; dt < kMaxDvTiles; ++dt) {
+      if (dt < ndt) {
+        ushort4 o4;
+        o4.x = f32_to_bf16(oacc[dt][0] * inv);
+        o4.y = f32_to_bf16(oacc[dt][1] * inv);
+        o4.z = f32_to_bf16(oacc[dt][2] * inv);
+        o4.w = f32_to_bf16(oacc[dt][3] * inv);
+        *(ushort4*)(op + dt * 16) = o4;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 static bool dense_heads3(const torch::Tensor& t) {
@@ -546,8 +794,41 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
                          (float)softcap, (int)chunk, (int)window, (float)out_scale,
                          (int)sink, H, G, D, Dv, bs);
     };
-    if (D <= 128 && Dv <= 256) launch(masked_prefill_mfma_kernel<8, 16>);
-    else launch(masked_prefill_mfma_kernel<32, 32>);
+    const size_t lds_shared =
+        (size_t)2 * (kKT * (D + kKPad) + Dv * (kKT + kVPad)) * sizeof(bf16raw);
+    const bool cache_al16 = ((size_t)k_cache.data_ptr()) % 16 == 0 &&
+                            ((size_t)v_cache.data_ptr()) % 16 == 0;
+    if (D <= 128 && Dv <= 256 && lds_shared <= 64 * 1024 && cache_al16) {
+      // tiles shared through LDS by up to 8 waves: heads of a group first,
+      // then neighbouring query tiles
+      const int rep = H / G;
+      int HW = 1;
+      while (HW * 2 <= rep && HW < 8) HW *= 2;
+      const int WPB = HW < 4 ? 4 : HW;
+      const int QW = WPB / HW;
+      const int btiles = (int)((max_len + QW * 16 - 1) / (QW * 16));
+      const int zb = (rep + HW - 1) / HW;
+      TORCH_CHECK(G <= 65535 && zb <= 65535);
+      auto launch_shared = [&](auto kern) {
+      hipLaunchKernelGGL(kern,
+                         dim3(n_seq * btiles, G, zb), dim3(WPB * WAVE), lds_shared,
+                         SEQ_STREAM(), (bf16raw*)out.data_ptr(), out.stride(0),
+                         (const bf16raw*)q.data_ptr(), q.stride(0),
+                         (const bf16raw*)k_cache.data_ptr(),
+                         (const bf16raw*)v_cache.data_ptr(),
+                         (const int*)block_tables.data_ptr(),
+                         (int)block_tables.size(1), (const int*)start_loc.data_ptr(),
+                         (const int*)positions.data_ptr(), btiles, (float)scale,
+                         (float)softcap, (int)chunk, (int)window, (float)out_scale,
+                         (int)sink, H, G, D, Dv, bs, HW, QW);
+      };
+      if (D % 32 == 0) launch_shared(masked_prefill_mfma_shared_kernel<8, 16, true>);
+      else launch_shared(masked_prefill_mfma_shared_kernel<8, 16, false>);
+    } else if (D <= 128 && Dv <= 256) {
+      launch(masked_prefill_mfma_kernel<8, 16>);
+    } else {
+      launch(masked_prefill_mfma_kernel<32, 32>);
+    }
     SEQ_CHECK_LAUNCH();
     return;
   }
