@@ -655,6 +655,193 @@ __global__ __launch_bounds__(512) void masked_prefill_mfma_shared_kernel(
   }
 }
 
+constexpr int kDW = 4;  // waves of a decode block; each takes every fourth key tile
+
+// Single decode tokens on the matrix cores, bf16. grid (T, G, ceil(rep / 16)):
+// the 16 rows of an MFMA tile are the query heads that share one key/value
+// head (all heads of a latent layer, the group of a grouped layer), so a key
+// or value row is loaded once for all of them. The four waves walk disjoint
+// 32-key tiles: K rows come straight from the cache as A operands, the V tile
+// is transposed through a wave-private LDS region, statistics are fp32 in the
+// base-2 domain, and the waves' partial results are joined through LDS.
+template <int kMaxDSteps, int kMaxDvTiles>
+__global__ __launch_bounds__(kDW * WAVE) void masked_decode_mfma_kernel(
+    bf16raw* __restrict__ out, int64_t out_stride, const bf16raw* __restrict__ q,
+    int64_t q_stride, const bf16raw* __restrict__ k_cache,
+    const bf16raw* __restrict__ v_cache, const int* __restrict__ block_tables,
+    int max_blocks, const int* __restrict__ token_seq,
+    const int* __restrict__ positions, float scale, float softcap, int chunk,
+    int window, float out_scale, int sink, int H, int G, int D, int Dv, int bs,
+    int n_split, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int col = lane & 15, grp = lane >> 4;
+  const int t = blockIdx.x, g = blockIdx.y, rep = H / G;
+  const int zt = blockIdx.z / n_split, sp = blockIdx.z % n_split;
+  const int h0 = g * rep + zt * 16;
+  const int nh = min(16, (g + 1) * rep - h0);
+  const int pos = positions[t];
+  const int* bt = block_tables + (size_t)token_seq[t] * max_blocks;
+  int lo = 0;
+  if (chunk > 0) lo = (pos / chunk) * chunk;
+  if (window > 0) lo = max(lo, pos - window + 1);
+  const int nks = D / 16, ndt = Dv / 16;
+  constexpr int vrow = kKT + kVPad;
+  bf16raw* vt = (bf16raw*)smem + (size_t)wave * Dv * vrow;
+  bf16x4 qf[kMaxDSteps];
+#pragma unroll
+  for (int ks = 0; ks < kMaxDSteps; ++ks)
+    if (ks < nks)
+      qf[ks] = col < nh ? *(const bf16x4*)(q + (size_t)t * q_stride + (h0 + col) * D +
+                                           ks * 16 + grp * 4)
+                        : (bf16x4){0, 0, 0, 0};
+  f32x4 oacc[kMaxDvTiles];
+#pragma unroll
+  for (int dt = 0; dt < kMaxDvTiles; ++dt) oacc[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  // the visible keys in 32-key tiles, dealt to the splits in contiguous shares
+  const int n_tiles = (pos - lo) / kKT + 1;
+  const int per_split = (n_tiles + n_split - 1) / n_split;
+  const int tile_end = min(n_tiles, (sp + 1) * per_split);
+  for (int tile = sp * per_split + wave; tile < tile_end; tile += kDW) {
+    const int j0 = lo + tile * kKT;
+    // V tile, transposed: lane takes key (v % 32), 16-byte chunk (v / 32)
+    for (int v = lane; v < kKT * (Dv / 8); v += WAVE) {
+      const int row = v % kKT, c = v / kKT;
+      const int j = min(j0 + row, pos);
+      const uint4 x = *(const uint4*)(v_cache +
+          (((int64_t)bt[j / bs] * G + g) * bs + j % bs) * Dv + c * 8);
+      const uint32_t wv[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        vt[(c * 8 + 2 * e) * vrow + row] = (bf16raw)(wv[e] & 0xffffu);
+        vt[(c * 8 + 2 * e + 1) * vrow + row] = (bf16raw)(wv[e] >> 16);
+      }
+    }
+    f32x4 sacc[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      sacc[sub] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      const int jk = min(j0 + sub * 16 + col, pos);
+      const bf16raw* kp =
+          k_cache + (((int64_t)bt[jk / bs] * G + g) * bs + jk % bs) * D + grp * 4;
+#pragma unroll
+      for (int ks = 0; ks < kMaxDSteps; ++ks)
+        if (ks < nks)
+          sacc[sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+              *(const bf16x4*)(kp + ks * 16), qf[ks], sacc[sub], 0, 0, 0);
+    }
+    // this lane: head `col`, keys j0 + sub * 16 + grp * 4 + i
+    float sc[8];
+    float mt = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = j0 + (e >> 2) * 16 + grp * 4 + (e & 3);
+      float x = sacc[e >> 2][e & 3] * scale;
+      if (softcap > 0.f) x = softcap * tanhf(x / softcap);
+      sc[e] = j <= pos ? x * kLog2e : -INFINITY;  // j >= lo holds for every tile
+      mt = fmaxf(mt, sc[e]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 16, WAVE));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, WAVE));
+    const float m_new = fmaxf(m, mt);  // finite: the tile's first key is visible
+    const float corr = __builtin_amdgcn_exp2f(m - m_new);
+    float pv[8];
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pv[e] = __builtin_amdgcn_exp2f(sc[e] - m_new);
+      ps += pv[e];
+    }
+    union { bf16x8 v; uint32_t u[4]; } pk;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pk.u[e] = cvt_pk_bf16(pv[2 * e], pv[2 * e + 1]);
+    l = l * corr + ps;
+    m = m_new;
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's LDS writes landed
+    __builtin_amdgcn_wave_barrier();
+    const bf16raw* vp = vt + col * vrow + grp * 4;
+#pragma unroll
+    for (int dt = 0; dt < kMaxDvTiles; ++dt) {
+      if (dt < ndt) {
+        const bf16x4 v0 = *(const bf16x4*)(vp + dt * 16 * vrow);
+        const bf16x4 v1 = *(const bf16x4*)(vp + dt * 16 * vrow + 16);
+        const bf16x8 vf = (bf16x8){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+        f32x4 a = oacc[dt];
+        a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
+        oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pk.v, a, 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // all lanes read the tile before it is rewritten
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  __syncthreads();  // the staging regions are reused for the join
+  float* cm = (float*)smem;            // [waves][16] running max (base 2)
+  float* cl = cm + kDW * 16;           // [waves][16] sums
+  float* co = cl + kDW * 16;           // [waves][16][Dv] unnormalised outputs
+  if (grp == 0) {
+    cm[wave * 16 + col] = m;
+    cl[wave * 16 + col] = l;
+  }
+#pragma unroll
+  for (int dt = 0; dt < kMaxDvTiles; ++dt)
+    if (dt < ndt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        co[((size_t)wave * 16 + col) * Dv + dt * 16 + grp * 4 + i] = oacc[dt][i];
+    }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < nh * Dv; idx += blockDim.x) {
+    const int hh = idx / Dv, d = idx % Dv;
+    float mx = -INFINITY;
+    for (int w = 0; w < kDW; ++w) mx = fmaxf(mx, cm[w * 16 + hh]);
+    float lsum = 0.f, a = 0.f;
+    for (int w = 0; w < kDW; ++w) {
+      const float mw = cm[w * 16 + hh];
+      const float wsc = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - mx);
+      lsum += cl[w * 16 + hh] * wsc;
+      a += co[((size_t)w * 16 + hh) * Dv + d] * wsc;
+    }
+    if (n_split == 1) {
+      if (sink) lsum += __builtin_amdgcn_exp2f(-mx);
+      stf(out + (size_t)t * out_stride + (h0 + hh) * Dv + d, a * out_scale / lsum);
+    } else {
+      // partial result of this split: [t][head][split] -> (max, sum), values
+      const size_t row = ((size_t)t * H + h0 + hh) * n_split + sp;
+      part_o[row * Dv + d] = a;
+      if (d == 0) {
+        part_ml[row * 2] = mx;
+        part_ml[row * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// Join of the key splits of masked_decode_mfma_kernel: grid (T, H).
+__global__ void decode_split_join_kernel(bf16raw* __restrict__ out, int64_t out_stride,
+                                         const float* __restrict__ part_o,
+                                         const float* __restrict__ part_ml, int H,
+                                         int Dv, int n_split, float out_scale,
+                                         int sink) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const size_t row0 = ((size_t)t * H + h) * n_split;
+  float mx = -INFINITY;
+  for (int s = 0; s < n_split; ++s) mx = fmaxf(mx, part_ml[(row0 + s) * 2]);
+  for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
+    float lsum = 0.f, a = 0.f;
+    for (int s = 0; s < n_split; ++s) {
+      const float ms = part_ml[(row0 + s) * 2];
+      if (ms == -INFINITY) continue;  // a split without keys wrote nothing usable
+      const float w = __builtin_amdgcn_exp2f(ms - mx);
+      lsum += part_ml[(row0 + s) * 2 + 1] * w;
+      a += part_o[(row0 + s) * Dv + d] * w;
+    }
+    if (sink) lsum += __builtin_amdgcn_exp2f(-mx);
+    stf(out + (size_t)t * out_stride + h * Dv + d, a * out_scale / lsum);
+  }
+}
+
 }  // namespace
 
 static bool dense_heads3(const torch::Tensor& t) {
@@ -828,6 +1015,51 @@ void masked_paged_attention(torch::Tensor out, torch::Tensor q,
       launch(masked_prefill_mfma_kernel<8, 16>);
     } else {
       launch(masked_prefill_mfma_kernel<32, 32>);
+    }
+    SEQ_CHECK_LAUNCH();
+    return;
+  }
+  // worth it when many heads share a row (measured: 16 heads on one latent
+  // 60 -> 28 us per call, groups of 4 no faster than the generic kernel)
+  if (q.scalar_type() == torch::kBFloat16 && max_len == 1 && H / G >= 8 && D % 16 == 0 &&
+      Dv % 16 == 0 && D <= 128 && Dv <= 128 && al8(q) &&
+      ((size_t)k_cache.data_ptr()) % 16 == 0 && ((size_t)v_cache.data_ptr()) % 16 == 0) {
+    // decode tokens: the heads of a key/value group are the rows of a tile
+    const int rep = H / G, zb = (rep + 15) / 16;
+    const size_t stage = (size_t)kDW * Dv * (kKT + kVPad) * sizeof(bf16raw);
+    const size_t join = (size_t)kDW * (32 + 16 * Dv) * sizeof(float);
+    // split the keys over blocks so that a wave walks about two tiles at the
+    // longest context the block tables can describe; splits beyond a
+    // sequence's keys exit at once
+    const int64_t cap = (int64_t)block_tables.size(1) * bs;
+    int n_split = (int)std::min<int64_t>(16, std::max<int64_t>(1, (cap + 255) / 256));
+    while (n_split > 1 && (int64_t)T * G * zb * n_split > 8192) n_split /= 2;
+    TORCH_CHECK(G <= 65535 && (int64_t)zb * n_split <= 65535);
+    torch::Tensor part_o, part_ml;
+    if (n_split > 1) {
+      auto f32 = torch::TensorOptions().dtype(torch::kFloat32).device(q.device());
+      part_o = torch::empty({(int64_t)T * H * n_split, Dv}, f32);
+      part_ml = torch::empty({(int64_t)T * H * n_split, 2}, f32);
+    }
+    hipLaunchKernelGGL((masked_decode_mfma_kernel<8, 8>), dim3(T, G, zb * n_split),
+                       dim3(kDW * WAVE), stage > join ? stage : join, SEQ_STREAM(),
+                       (bf16raw*)out.data_ptr(), out.stride(0),
+                       (const bf16raw*)q.data_ptr(), q.stride(0),
+                       (const bf16raw*)k_cache.data_ptr(),
+                       (const bf16raw*)v_cache.data_ptr(),
+                       (const int*)block_tables.data_ptr(), (int)block_tables.size(1),
+                       (const int*)token_seq.data_ptr(), (const int*)positions.data_ptr(),
+                       (float)scale, (float)softcap, (int)chunk, (int)window,
+                       (float)out_scale, (int)sink, H, G, D, Dv, bs, n_split,
+                       n_split > 1 ? (float*)part_o.data_ptr() : nullptr,
+                       n_split > 1 ? (float*)part_ml.data_ptr() : nullptr);
+    if (n_split > 1) {
+      SEQ_CHECK_LAUNCH();
+      hipLaunchKernelGGL(decode_split_join_kernel, dim3(T, H), dim3(64), 0, SEQ_STREAM(),
+                         (bf16raw*)out.data_ptr(), out.stride(0),
+                         (const float*)part_o.data_ptr(),
+                         (const float*)part_ml.data_ptr(), H, (int)Dv, n_split,
+                         (float)out_scale, (int)sink);
     }
     SEQ_CHECK_LAUNCH();
     return;

@@ -783,3 +783,40 @@ def test_kernel_head_linear(dtype, T, H, A, B):
 
         _, c, _, gg = _both(run, wide, w, gate)
         assert (c.float() - gg.cpu().float()).abs().max() < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv,shared", [(16, 1, 128, 128, True), (16, 2, 32, 16, False),
+                                             (20, 1, 48, 48, True), (4, 4, 64, 64, False),
+                                             (9, 1, 16, 128, False)])
+def test_kernel_decode_attention_grouped_heads(H, G, D, Dv, shared):
+    """Pure decode steps in bf16 with eight or more heads per key/value head
+    take the kernel whose tile rows are the heads of a group (keys split over
+    blocks, joined by a second kernel); contexts around the 32-key tile and
+    the split borders, with and without window and sink."""
+    g = torch.Generator().manual_seed(H + D)
+    bs, lens = 16, [1, 31, 32, 33, 127, 128, 129, 200, 1000]
+    nb = sum((n + bs - 1) // bs for n in lens) + 2
+    perm = torch.randperm(nb, generator=g).tolist()
+    kc = (torch.randn(nb, G, bs, D, generator=g) * 0.5).bfloat16()
+    vc = kc if shared else torch.randn(nb, G, bs, Dv, generator=g).bfloat16()
+    width = max((n + bs - 1) // bs for n in lens)
+    tables, at = [], 0
+    for n in lens:
+        k = (n + bs - 1) // bs
+        tables.append(perm[at : at + k] + [0] * (width - k))
+        at += k
+    runs = [(1, -1)] * len(lens)
+    positions = [n - 1 for n in lens]
+    q = torch.randn(len(lens), H, D, generator=g).bfloat16()
+    for window, sink in [(0, False), (0, True), (40, True), (1, False)]:
+        outs = []
+        for dev in ("cpu", "cuda"):
+            meta = sops.SeqMeta.build(runs, torch.tensor(positions, dtype=torch.int32).to(dev),
+                                      dev, block_tables=torch.tensor(tables, dtype=torch.int32).to(dev))
+            out = torch.zeros(len(lens), H, Dv, dtype=torch.bfloat16, device=dev)
+            kcd = kc.to(dev)
+            sops.masked_paged_attention(q.to(dev), kcd, kcd if shared else vc.to(dev), meta,
+                                        D ** -0.5, out, window=window, sink=sink)
+            outs.append(out.float().cpu())
+        assert (outs[0] - outs[1]).abs().max() < 5e-2, (window, sink)
