@@ -122,6 +122,7 @@ class LLMEngine:
     ) -> Request:
         if params is None:
             params = SamplingParams()
+        self._check_token_ids(prompt_token_ids)
         if not params.ignore_eos and self.arch.eos_token_id not in params.stop_token_ids:
             params = dataclasses.replace(
                 params,
@@ -174,6 +175,16 @@ class LLMEngine:
             )
         self.scheduler.add_request(req)
         return req
+
+    def _check_token_ids(self, token_ids) -> None:
+        """Token ids index the embedding table on the GPU: an id outside the
+        vocabulary is rejected here, on the host."""
+        if len(token_ids) and not (
+            0 <= min(token_ids) and max(token_ids) < self.arch.vocab_size
+        ):
+            raise RequestError(
+                f"token id outside the vocabulary [0, {self.arch.vocab_size})"
+            )
 
     def abort_request(self, request_id: str) -> None:
         self.scheduler.abort(request_id)
@@ -245,6 +256,7 @@ class LLMEngine:
         """
         chunks, want = [], {}
         for rid, toks, w in entries:
+            self._check_token_ids(toks)
             req = self._fixed.get(rid)
             if req is None:
                 req = Request(list(toks), SamplingParams(ignore_eos=True),

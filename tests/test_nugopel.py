@@ -516,6 +516,17 @@ def test_unconsumed_tensor_is_an_error(tmp_path):
         engine(d, "cpu")
 
 
+def test_token_ids_outside_the_vocabulary_are_rejected(tmp_path):
+    cfg = config([lat(mlp=None)])
+    d, _ = model_dir(tmp_path, cfg, seed=21)
+    eng = engine(d, "cpu")
+    with pytest.raises(ValueError):
+        eng.step_fixed([("a", [1, cfg["vocab"]], [0])])
+    with pytest.raises(ValueError):
+        eng.add_request([3, -1])
+    assert eng.step_fixed([("b", [1, cfg["vocab"] - 1], [1])], ["b"])[0].shape[0] == 1
+
+
 def test_latent_source_must_cache_a_latent(tmp_path):
     cfg = config([attn(), lat(kv_from=0)])
     d, _ = model_dir(tmp_path, cfg, seed=17, W={"embed": torch.zeros(1).bfloat16()})
